@@ -74,6 +74,15 @@ __global__ __launch_bounds__(64 * (WM * WN * KG + LW)) void gemm_glds_kernel(con
         p.a = reinterpret_cast<const char*>(p.a) + (int64_t) blockIdx.y * p.batch_a;
         p.w = reinterpret_cast<const char*>(p.w) + (int64_t) blockIdx.y * p.batch_w;
         p.c = reinterpret_cast<char*>(p.c) + (int64_t) blockIdx.y * p.batch_c;
+        if (p.group_off)
+        {
+            const int64_t o = p.group_off[blockIdx.y];
+            p.M = p.group_off[blockIdx.y + 1] - (int) o;
+            if (p.M <= 0)
+                return;
+            p.a = reinterpret_cast<const char*>(p.a) + o * p.lda * 2;
+            p.c = reinterpret_cast<char*>(p.c) + o * p.ldc * (p.out_dtype == DT_FLOAT ? 4 : 2);
+        }
     }
     constexpr bool SQ = WT == W_INT8_SQ;
     constexpr int ES = SQ ? 1 : 2; // bytes per A / W element
@@ -114,6 +123,11 @@ __global__ __launch_bounds__(64 * (WM * WN * KG + LW)) void gemm_glds_kernel(con
     const int tm = wg % tiles_m, tn = wg / tiles_m; // M fastest: the (few) row panels of one W panel run together
     const int m0 = tm * BM, n0 = tn * BN;
     const int M = p.M, N = p.N;
+    if constexpr (WT == W_BF16)
+    {
+        if (n0 >= N)
+            return; // a group with fewer rows than the launch's bound has fewer tiles than the grid
+    }
     const int ntile = (p.K * ES) / BKB;
 
     // ---- DMA source addresses: chunk c (RPC tile rows) -> lane l: row c * RPC + l / PPR, LDS piece l % PPR

@@ -366,6 +366,9 @@ struct GemmParams
     // w + b * batch_w, c + b * batch_c (no resid / residual)
     int32_t batch = 1;
     int64_t batch_a = 0, batch_w = 0, batch_c = 0;
+    // ... grouped: device int32 [batch + 1]; product b takes rows [group_off[b], group_off[b + 1]) of a and c (batch_a = batch_c = 0), M
+    // is the host's bound on a group's rows
+    const int32_t* group_off = nullptr;
     // microbench hook (tllm_gemm_set_clock_probe), set by the launchers only: 2 x uint64 per workgroup {shader cycles, 100 MHz ticks}
     void* clock_probe = nullptr;
     // split-K-2 forms of gemm_sqp.hip (r06), set by the launcher only: per tile two slabs of AH x BN accumulators + two flag words

@@ -72,6 +72,15 @@ __device__ __forceinline__ StackGemmParams batch_slice(StackGemmParams p)
     p.w = reinterpret_cast<const char*>(p.w) + b * p.stride_w * ES;
     if (p.c)
         p.c = reinterpret_cast<char*>(p.c) + b * p.stride_c * ((p.out_f32 || DT == DT_FLOAT) ? 4 : 2);
+    if (p.group_off)
+    {
+        // grouped form: this product's rows are a range of a and c that the device knows
+        const int64_t o = p.group_off[b];
+        p.M = p.group_off[b + 1] - (int) o;
+        p.a = reinterpret_cast<const char*>(p.a) + o * p.lda * ES;
+        if (p.c)
+            p.c = reinterpret_cast<char*>(p.c) + o * p.ldc * ((p.out_f32 || DT == DT_FLOAT) ? 4 : 2);
+    }
     return p;
 }
 
@@ -85,6 +94,8 @@ __global__ __launch_bounds__(256) void fma_tile_kernel(const StackGemmParams p_i
     __shared__ float Ws[TK][TN + 4];
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+    if (m0 >= p.M)
+        return; // (a group with fewer rows than the launch's bound)
     float acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -139,7 +150,7 @@ __global__ __launch_bounds__(256) void skinny_kernel(const StackGemmParams p_in)
     const StackGemmParams p = batch_slice<DT_BF16>(p_in);
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     const int n0 = (blockIdx.x * 4 + wid) * SK_R;
-    if (n0 >= p.N)
+    if (n0 >= p.N || p.M <= 0)
         return;
     float acc[SK_R][MR];
 #pragma unroll
@@ -245,9 +256,9 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
         set_error("stack_gemm: element type %d is not served (bfloat16 or float32)", p.dtype);
         return -1;
     }
-    if (p.batch < 1 || (p.batch > 1 && p.resid))
+    if (p.batch < 1 || (p.batch > 1 && p.resid) || (p.group_off && (p.resid || p.stride_a || p.stride_c)))
     {
-        set_error("stack_gemm: batch %d (a batched product has no residual seam)", p.batch);
+        set_error("stack_gemm: batch %d (a batched product has no residual seam; a grouped one takes its rows from one a and one c)", p.batch);
         return -1;
     }
     const dim3 tiles((p.N + TN - 1) / TN, (p.M + TM - 1) / TM, p.batch);
@@ -269,10 +280,11 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
             hipLaunchKernelGGL((skinny_kernel<8>), grid, dim3(256), 0, stream, p);
         return launched("stack_gemm skinny");
     }
-    if (aligned)
+    if (aligned && (!p.group_off || p.K % 64 == 0))
     {
-        // the LDS-DMA tiles take a batch in one launch (blockIdx.y); the register-staged tiles one product per launch
-        const bool glds = p.M >= 32 && p.K % 64 == 0;
+        // the LDS-DMA tiles take a batch in one launch (blockIdx.y); the register-staged tiles one product per launch (and no
+        // groups: their row count is the device's)
+        const bool glds = (p.M >= 32 || p.group_off) && p.K % 64 == 0;
         const int launches = glds ? 1 : p.batch;
         int rc = 0;
         for (int b = 0; b < launches && rc == 0; ++b)
@@ -302,6 +314,7 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
                 g.batch_a = p.stride_a * 2;
                 g.batch_w = p.stride_w * 2;
                 g.batch_c = p.stride_c * (p.out_f32 ? 4 : 2);
+                g.group_off = p.group_off;
                 rc = launch_glds_bf16(g, stream);
             }
             else

@@ -1,7 +1,7 @@
 // Host-side launch interface of the kernels behind the ragged-batch stack engine (runtime/stack_engine.cpp): decoder
 // stacks whose layers are described at run time (grouped RMS norms, gated residuals or hyper-connected residual streams, looped
 // layer ranges, attention over a paged cache in its variants - differential maps, masks, distance penalties, sigmoid weights, sinks,
-// a shared latent -, HGRN2 recurrences over per-sequence state slots).
+// a shared latent -, HGRN2 and selective state-space recurrences over per-sequence state slots, routed mixtures of experts).
 //
 // A step is one packed batch of `tokens` rows: portions of prompts and single decoded tokens of several sequences side
 // by side.  Row t belongs to batch entry tok_entry[t] and sits at position tok_pos[t] of its sequence.  Every kernel is
@@ -50,6 +50,9 @@ struct StackGemmParams
     int32_t act = ACT_NONE;           // (no resid)
     int32_t batch = 1;
     int64_t stride_a = 0, stride_w = 0, stride_c = 0; // elements, between the operands of consecutive products
+    // Grouped form of a batch (a mixture of experts): device int32 [batch + 1]; product b takes rows [group_off[b], group_off[b + 1]) of
+    // a and c (stride_a = stride_c = 0) and weight block b; M is the host's bound on the rows of one group.
+    const int32_t* group_off = nullptr;
 };
 int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream);
 
@@ -92,8 +95,14 @@ struct StackHyperParams
     const int32_t* rows = nullptr; // [tokens] or null
 };
 int launch_stack_hyper_norm(const StackHyperParams& p, hipStream_t stream);
-// y[t, c] = gelu_tanh(gu[t, c]) * gu[t, ff + c] over a [tokens, ld] projection that holds gate then up columns
-int launch_stack_gelu_gate(void* y, const void* gu, int32_t dtype, int32_t tokens, int32_t ff, int64_t ld, hipStream_t stream);
+// y[t, c] = act(gu[t, c]) * gu[t, ff + c] over a [tokens, ld] projection that holds gate then up columns; act: GATE_GELU_TANH | GATE_SILU
+constexpr int32_t GATE_GELU_TANH = 0, GATE_SILU = 1;
+int launch_stack_gelu_gate(void* y, const void* gu, int32_t dtype, int32_t tokens, int32_t ff, int64_t ld, hipStream_t stream,
+    int32_t act = GATE_GELU_TANH);
+// y[r, :n] = x[r, :n] / sqrt(mean(x[r, :n]^2) + eps) * w over rows of the element type with their own strides (a low-rank latent
+// inside a wider projection); one wave per row
+int launch_stack_row_rmsnorm(void* y, int64_t ldy, const void* x, int64_t ldx, const float* w, int32_t dtype, int32_t rows, int32_t n, float eps,
+    hipStream_t stream);
 
 // ---------------------------------------------------------------------------------------------
 // Rotary positions: pair (2i, 2i + 1) of the first `dims` dimensions of every map of every head, angle = pos * freq[i]
@@ -107,6 +116,7 @@ struct StackAttnParams
     int32_t tokens = 0, entries = 0;
     int32_t heads = 0, kv_heads = 0, maps = 1, dim = 0, vdim = 0;
     int32_t rot_dims = 0;
+    int32_t rot_halves = 0;      // latent_prep: 0 pairs (2i, 2i + 1), 1 pairs (i, i + rot_dims / 2)
     const float* freq = nullptr; // fp32 [rot_dims / 2], device
     float mscale = 1.f;
     float scale = 1.f, softcap = 0.f; // score = softcap * tanh(q.k * scale / softcap) when softcap > 0
@@ -170,9 +180,12 @@ float stack_rope_freqs(float* freq, int32_t dims, double base, double factor, do
 // launch_stack_gemm calls.  proj [tokens, ldp]: q (heads * (dim + rot): per head plain then rotated part), then rank + rot columns.
 // It writes the rotated q part into q_abs[t, h, rank : rank + rot] and appends the token to the cache; a.dim = rank + rot,
 // a.vdim = rank, a.kv_heads = 1, a.rot_dims = how many of the rot dimensions turn (pairs (2i, 2i + 1), the rest pass), a.freq,
-// a.q = q_abs and the pools are read from `a`.
+// a.q = q_abs and the pools are read from `a`; a.rot_halves chooses the pairing, a.mscale multiplies cos and sin.  Where the
+// queries come from a projection of their own (a query latent), q_src [tokens, ldq] holds them and dkv_col is the column of proj at
+// which the rank + rot columns start.
 // ---------------------------------------------------------------------------------------------
-int launch_stack_latent_prep(const StackAttnParams& a, int32_t qk_dim, const float* latent_norm_w, hipStream_t stream);
+int launch_stack_latent_prep(const StackAttnParams& a, int32_t qk_dim, const float* latent_norm_w, hipStream_t stream,
+    const void* q_src = nullptr, int64_t ldq = 0, int32_t dkv_col = -1);
 
 // ---------------------------------------------------------------------------------------------
 // HGRN2: per head a state S [dim, vdim] (fp32, one per sequence slot), S <- diag(f) S + (1 - f) v^T, o = S^T q with
@@ -201,6 +214,73 @@ struct StackHgrnParams
 };
 int launch_stack_hgrn2(const StackHgrnParams& p, hipStream_t stream);
 bool stack_hgrn2_serves(int32_t dim, int32_t vdim); // shapes one of its two forms takes
+
+// ---------------------------------------------------------------------------------------------
+// Selective state-space layer (Mamba-2): proj [tokens, ldp] = [z: inner | x: inner | B: groups * state | C: groups * state |
+// dt: heads], inner = heads * vdim.  x, B, C pass a causal convolution over `taps` tokens per channel (conv_w [channels, taps], the
+// last column meets the current token; bias) and silu: launch_stack_ssm_conv writes them to xbc [tokens, channels] and moves the
+// sequence's last taps - 1 raw inputs into conv_state [slots, taps - 1, channels].  launch_stack_ssm_scan: per head h (reading group
+// h / (heads / groups)), with dt = softplus(dt + dt_bias[h]):
+//   S <- exp(-exp(a_log[h]) dt) S + dt B x^T   (S [state, vdim], fp32, one per slot),   y = S^T C + d_skip[h] x,
+// and y32 [tokens, inner] = y * silu(z) in fp32 (the grouped norm behind it is launch_stack_group_rmsnorm).  An entry whose pos0 is 0
+// starts from zero state and zero convolution inputs.
+// ---------------------------------------------------------------------------------------------
+struct StackSsmParams
+{
+    int32_t dtype = DT_BF16;
+    int32_t tokens = 0, entries = 0;
+    int32_t heads = 0, vdim = 0, state = 0, groups = 1, taps = 0;
+    const void* proj = nullptr;
+    int64_t ldp = 0;
+    const float* conv_w = nullptr; // [channels, taps]
+    const float* conv_b = nullptr; // [channels]
+    const float* dt_bias = nullptr; // [heads]
+    const float* a_log = nullptr;   // [heads]
+    const float* d_skip = nullptr;  // [heads]
+    float* conv_state = nullptr;    // [slots, taps - 1, channels]
+    float* ssm_state = nullptr;     // [slots, heads, state, vdim]
+    void* xbc = nullptr;            // scratch [tokens, channels], element type
+    float* y32 = nullptr;           // [tokens, inner]
+    const int32_t* tok_entry = nullptr;
+    const int32_t* tok_pos = nullptr;
+    const int32_t* ent_slot = nullptr;
+    const int32_t* ent_first = nullptr;
+    const int32_t* ent_count = nullptr;
+    const int32_t* ent_pos0 = nullptr;
+};
+int launch_stack_ssm_conv(const StackSsmParams& p, hipStream_t stream);
+int launch_stack_ssm_scan(const StackSsmParams& p, hipStream_t stream);
+bool stack_ssm_serves(int32_t vdim, int32_t state, int32_t taps);
+
+// ---------------------------------------------------------------------------------------------
+// Routed mixture of experts.  Router: z = router_w h in fp32 over experts + identity outputs, s = softmax(z); the choice is made on
+// s + correction among the experts of the group_keep groups (of group_count equal groups of neighbours) whose largest such value is
+// largest, `top` of them; a chosen expert's weight is s * scale (without the correction, not renormalised).  The last `identity`
+// outputs are experts without weights that return h.
+//   launch_stack_moe_route   -> topk_idx / topk_w [tokens, top]
+//   launch_stack_moe_sort    -> group_off [experts + 1], slot_of_pair [tokens * top] (-1: identity), a_sorted: the rows of h in
+//                               expert order, one per (token, chosen expert); the grouped products (launch_stack_gemm, group_off) run on them
+//   launch_stack_moe_combine -> y[t, :] = sum_k w_k * (expert: y_sorted[slot_k, :] | identity: h[t, :]), fp32
+// ---------------------------------------------------------------------------------------------
+struct StackMoeParams
+{
+    int32_t dtype = DT_BF16;
+    int32_t tokens = 0, width = 0;
+    int32_t experts = 0, identity = 0, top = 0, group_count = 1, group_keep = 1;
+    float scale = 1.f;
+    const void* h = nullptr;          // [tokens, width]
+    const float* router_w = nullptr;  // [experts + identity, width]
+    const float* correction = nullptr; // [experts + identity] or null
+    int32_t* topk_idx = nullptr;
+    float* topk_w = nullptr;
+    int32_t* group_off = nullptr;
+    int32_t* slot_of_pair = nullptr;
+    int32_t* pair_of_slot = nullptr;  // [tokens * top], -1 behind the last used slot
+    void* a_sorted = nullptr;         // [tokens * top, width]
+};
+int launch_stack_moe_route(const StackMoeParams& p, hipStream_t stream);
+int launch_stack_moe_sort(const StackMoeParams& p, hipStream_t stream);
+int launch_stack_moe_combine(const StackMoeParams& p, const float* y_sorted, float* y, hipStream_t stream);
 
 } // namespace kernels
 } // namespace tllm

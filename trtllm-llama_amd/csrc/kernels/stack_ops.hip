@@ -214,17 +214,36 @@ __device__ __forceinline__ float gelu_tanh(float z)
 }
 
 template <int DT>
-__global__ __launch_bounds__(256) void gelu_gate_kernel(void* y, const void* gu, int tokens, int ff, int64_t ld)
+__global__ __launch_bounds__(256) void gelu_gate_kernel(void* y, const void* gu, int tokens, int ff, int64_t ld, int act)
 {
     const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (int64_t) tokens * ff)
         return;
     const int t = (int) (i / ff), c = (int) (i % ff);
     const float g = El<DT>::ld(gu, (int64_t) t * ld + c), u = El<DT>::ld(gu, (int64_t) t * ld + ff + c);
-    float a = gelu_tanh(g);
+    float a = act == GATE_SILU ? g / (1.f + expf(-g)) : gelu_tanh(g);
     if (DT == DT_BF16)
         a = bf2f(f2bf(a)); // the activation is a bfloat16 value before it meets the other branch
     El<DT>::st(y, i, a * u);
+}
+
+// one wave per row: y = x / sqrt(mean(x^2) + eps) * w over n elements of the element type, rows with their own strides
+template <int DT>
+__global__ __launch_bounds__(256) void row_rmsnorm_kernel(void* y, int64_t ldy, const void* x, int64_t ldx, const float* w, int rows, int n,
+    float eps)
+{
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (r >= rows)
+        return;
+    float ss = 0.f;
+    for (int c = lane; c < n; c += 64)
+    {
+        const float v = El<DT>::ld(x, (int64_t) r * ldx + c);
+        ss += v * v;
+    }
+    const float inv = 1.f / sqrtf(wave_sum(ss) / (float) n + eps);
+    for (int c = lane; c < n; c += 64)
+        El<DT>::st(y, (int64_t) r * ldy + c, El<DT>::ld(x, (int64_t) r * ldx + c) * inv * w[c]);
 }
 
 // --------------------------------------------------------------------------------------------------- rotary + cache append
@@ -341,7 +360,8 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const StackAttnParams p)
 // the page ([c | k_rot] as the key row, c channel-major as the value row), and the rotation of every head's rotated query part into
 // the absorbed query [a | q_rot] (the `a` part is a product of its own).  One wave per (row, head) plus one per row for the latent.
 template <int DT>
-__global__ __launch_bounds__(256) void latent_prep_kernel(const StackAttnParams p, int qk_dim, const float* norm_w)
+__global__ __launch_bounds__(256) void latent_prep_kernel(const StackAttnParams p, int qk_dim, const float* norm_w, const void* q_src,
+    int64_t ldq, int dkv_col)
 {
     const int t = blockIdx.x, lane = threadIdx.x & 63;
     const int vec = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -349,26 +369,34 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const StackAttnParams 
         return;
     const int C = p.vdim, R = p.dim - C, pos = p.tok_pos[t]; // of the R dimensions of the rotated part the first rot_dims turn
     const int64_t row = (int64_t) t * p.ldp;
+    const int half = p.rot_dims >> 1;
+    // dimension d < rot_dims of a rotated part: its partner, its frequency, and whether it is the second of its pair
+    auto turn = [&](const void* base, int64_t src, int d) -> float {
+        float x = El<DT>::ld(base, src + d);
+        if (d < p.rot_dims)
+        {
+            const int partner = p.rot_halves ? (d < half ? d + half : d - half) : (d ^ 1);
+            const int fi = p.rot_halves ? (d < half ? d : d - half) : (d >> 1);
+            const bool second = p.rot_halves ? d >= half : (d & 1);
+            const float other = El<DT>::ld(base, src + partner);
+            float sn, cs;
+            sincosf((float) pos * p.freq[fi], &sn, &cs);
+            sn *= p.mscale;
+            cs *= p.mscale;
+            x = second ? x * cs + other * sn : x * cs - other * sn;
+        }
+        return x;
+    };
     if (vec < p.heads)
     {
-        const int64_t src = row + (int64_t) vec * (qk_dim + R) + qk_dim;
+        const int64_t src = (int64_t) t * ldq + (int64_t) vec * (qk_dim + R) + qk_dim;
         for (int d = lane; d < R; d += 64)
-        {
-            float x = El<DT>::ld(p.proj, src + d);
-            if (d < p.rot_dims)
-            {
-                const float other = El<DT>::ld(p.proj, src + (d ^ 1));
-                float sn, cs;
-                sincosf((float) pos * p.freq[d >> 1], &sn, &cs);
-                x = (d & 1) ? x * cs + other * sn : x * cs - other * sn;
-            }
-            El<DT>::st(p.q, ((int64_t) t * p.heads + vec) * p.dim + C + d, x);
-        }
+            El<DT>::st(p.q, ((int64_t) t * p.heads + vec) * p.dim + C + d, turn(q_src, src, d));
         return;
     }
     const int e = p.tok_entry[t];
     const int blk = p.block_table[(int64_t) e * p.max_blocks + pos / p.page], off = pos % p.page;
-    const int64_t src = row + (int64_t) p.heads * (qk_dim + R);
+    const int64_t src = row + dkv_col;
     float ss = 0.f;
     for (int c = lane; c < C; c += 64)
     {
@@ -384,17 +412,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const StackAttnParams 
         El<DT>::st(p.v_pool, ((int64_t) blk * C + c) * p.page + off, x);
     }
     for (int d = lane; d < R; d += 64)
-    {
-        float x = El<DT>::ld(p.proj, src + C + d);
-        if (d < p.rot_dims)
-        {
-            const float other = El<DT>::ld(p.proj, src + C + (d ^ 1));
-            float sn, cs;
-            sincosf((float) pos * p.freq[d >> 1], &sn, &cs);
-            x = (d & 1) ? x * cs + other * sn : x * cs - other * sn;
-        }
-        El<DT>::st(p.k_pool, krow + C + d, x);
-    }
+        El<DT>::st(p.k_pool, krow + C + d, turn(p.proj, src + C, d));
 }
 
 // ------------------------------------------------------------------------------------------------ attention, general form
@@ -1002,7 +1020,7 @@ int launch_stack_group_rmsnorm(void* y1, void* y2, const float* x, const int32_t
     return launched("stack_group_rmsnorm");
 }
 
-int launch_stack_gelu_gate(void* y, const void* gu, int32_t dtype, int32_t tokens, int32_t ff, int64_t ld, hipStream_t stream)
+int launch_stack_gelu_gate(void* y, const void* gu, int32_t dtype, int32_t tokens, int32_t ff, int64_t ld, hipStream_t stream, int32_t act)
 {
     const int64_t n = (int64_t) tokens * ff;
     if (n <= 0)
@@ -1011,10 +1029,25 @@ int launch_stack_gelu_gate(void* y, const void* gu, int32_t dtype, int32_t token
         return -1;
     const dim3 grid((unsigned) ((n + 255) / 256));
     if (dtype == DT_BF16)
-        hipLaunchKernelGGL((gelu_gate_kernel<DT_BF16>), grid, dim3(256), 0, stream, y, gu, tokens, ff, ld);
+        hipLaunchKernelGGL((gelu_gate_kernel<DT_BF16>), grid, dim3(256), 0, stream, y, gu, tokens, ff, ld, act);
     else
-        hipLaunchKernelGGL((gelu_gate_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, y, gu, tokens, ff, ld);
+        hipLaunchKernelGGL((gelu_gate_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, y, gu, tokens, ff, ld, act);
     return launched("stack_gelu_gate");
+}
+
+int launch_stack_row_rmsnorm(void* y, int64_t ldy, const void* x, int64_t ldx, const float* w, int32_t dtype, int32_t rows, int32_t n, float eps,
+    hipStream_t stream)
+{
+    if (rows <= 0 || n <= 0)
+        return 0;
+    if (!known_dtype(dtype, "stack_row_rmsnorm"))
+        return -1;
+    const dim3 grid((rows + 3) / 4);
+    if (dtype == DT_BF16)
+        hipLaunchKernelGGL((row_rmsnorm_kernel<DT_BF16>), grid, dim3(256), 0, stream, y, ldy, x, ldx, w, rows, n, eps);
+    else
+        hipLaunchKernelGGL((row_rmsnorm_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, y, ldy, x, ldx, w, rows, n, eps);
+    return launched("stack_row_rmsnorm");
 }
 
 static bool attn_shape_ok(const StackAttnParams& p, const char* what)
@@ -1078,8 +1111,16 @@ int launch_stack_rope_kv(const StackAttnParams& p, hipStream_t stream)
     return launched("stack_rope_kv");
 }
 
-int launch_stack_latent_prep(const StackAttnParams& p, int32_t qk_dim, const float* latent_norm_w, hipStream_t stream)
+int launch_stack_latent_prep(const StackAttnParams& p, int32_t qk_dim, const float* latent_norm_w, hipStream_t stream, const void* q_src,
+    int64_t ldq, int32_t dkv_col)
 {
+    if (!q_src)
+    {
+        q_src = p.proj;
+        ldq = p.ldp;
+    }
+    if (dkv_col < 0)
+        dkv_col = p.heads * (qk_dim + (p.dim - p.vdim));
     if (p.tokens <= 0)
         return 0;
     if (!attn_shape_ok(p, "stack_latent_prep"))
@@ -1092,9 +1133,9 @@ int launch_stack_latent_prep(const StackAttnParams& p, int32_t qk_dim, const flo
     }
     const dim3 grid(p.tokens, (p.heads + 1 + 3) / 4);
     if (p.dtype == DT_BF16)
-        hipLaunchKernelGGL((latent_prep_kernel<DT_BF16>), grid, dim3(256), 0, stream, p, qk_dim, latent_norm_w);
+        hipLaunchKernelGGL((latent_prep_kernel<DT_BF16>), grid, dim3(256), 0, stream, p, qk_dim, latent_norm_w, q_src, ldq, dkv_col);
     else
-        hipLaunchKernelGGL((latent_prep_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, p, qk_dim, latent_norm_w);
+        hipLaunchKernelGGL((latent_prep_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, p, qk_dim, latent_norm_w, q_src, ldq, dkv_col);
     return launched("stack_latent_prep");
 }
 

@@ -46,12 +46,14 @@ enum MixerKind
 {
     MIX_ATTENTION = 0,
     MIX_HGRN2 = 1,
-    MIX_LATENT = 2
+    MIX_LATENT = 2,
+    MIX_MAMBA2 = 3
 };
 enum MlpKind
 {
     MLP_GELU_GATE = 0, // W_down (gelu_tanh(W_gate h) * W_up h)
-    MLP_RELU2 = 1      // W_down relu(W_up h)^2
+    MLP_RELU2 = 1,     // W_down relu(W_up h)^2
+    MLP_MOE = 2        // routed experts W_down (silu(W_gate h) * W_up h) of size ff, the last `identity` router outputs return h
 };
 struct HyperW
 {
@@ -75,11 +77,18 @@ struct Layer
     int kv_rank = 0, rot_part = 0;  // latent attention: rank of the latent, size of the shared rotated key part (rot_dims of it turn)
     int n_gate = 0, n_rg = 0;       // further columns of P1: per-head output gates, the gated residual's projection
     int n_lat = 0;                  // latent attention: heads * kv_rank
+    int q_rank = 0, rot_halves = 0; // latent attention: rank of a query latent (0: queries straight from the input), half-split pairs
+    int weights_of = -1;            // the layer whose weights this one runs on (its cache / state is its own)
+    int groups = 1, taps = 0, ssm_norm_groups = 1, n_conv = 0; // mamba2 (dim = state rows): B / C groups, convolution taps, parts of the output norm
+    int experts = 0, identity = 0, top = 0, route_groups = 1, route_keep = 1; // moe
+    double route_scale = 1;
     // device
     void *w_mix = nullptr, *w_o = nullptr, *w_gu = nullptr, *w_down = nullptr, *w_ukT = nullptr, *w_uv = nullptr;
     float *norm1 = nullptr, *norm2 = nullptr, *rg1_b = nullptr, *rg2_b = nullptr, *f_bias = nullptr, *lower = nullptr, *hnorm = nullptr,
           *freq = nullptr, *bias = nullptr, *temp = nullptr, *slope = nullptr, *r1 = nullptr, *r2 = nullptr, *sinkv = nullptr, *wbias = nullptr,
-          *lat_norm = nullptr;
+          *lat_norm = nullptr, *cq_norm = nullptr, *conv_w = nullptr, *conv_b = nullptr, *dt_bias = nullptr, *a_log = nullptr,
+          *d_skip = nullptr, *router_w = nullptr, *correction = nullptr;
+    void* w_uq = nullptr;
     HyperW hc[2];
 };
 
@@ -88,7 +97,8 @@ struct Run
     int layer = 0, pass = 0;
     bool enters_pass = false;
     void *k_pool = nullptr, *v_pool = nullptr; // attention
-    float* state = nullptr;                    // hgrn2
+    float* state = nullptr;                    // hgrn2, mamba2
+    float* conv_state = nullptr;               // mamba2: the last taps - 1 inputs of the convolution
 };
 
 } // namespace
@@ -116,7 +126,10 @@ struct tllm_stack
     float *x = nullptr, *x0 = nullptr, *o32 = nullptr, *logits = nullptr, *tap = nullptr, *y32 = nullptr;
     void *h1 = nullptr, *h2 = nullptr, *proj = nullptr, *q = nullptr, *ctx = nullptr, *act = nullptr, *hw = nullptr, *lat = nullptr;
     int32_t *ints = nullptr, *ids_out = nullptr, *pinned = nullptr;
-    int max_proj = 0, max_q = 0, max_ctx = 0, max_ff = 0, max_lat = 0;
+    void *xbc = nullptr, *cq = nullptr, *qfull = nullptr, *moe_a = nullptr;
+    float *moe_y = nullptr, *moe_w = nullptr;
+    int32_t* moe_i = nullptr;
+    int max_proj = 0, max_q = 0, max_ctx = 0, max_ff = 0, max_lat = 0, max_conv = 0, max_qrank = 0, max_qfull = 0, max_top = 0, max_experts = 0;
     int tap_tokens = 0;
 
     ~tllm_stack()
@@ -129,13 +142,16 @@ struct tllm_stack
     }
     void free_scratch()
     {
-        void* all[] = {x, x0, o32, logits, tap, y32, h1, h2, proj, q, ctx, act, hw, lat, ints, ids_out};
+        void* all[] = {x, x0, o32, logits, tap, y32, h1, h2, proj, q, ctx, act, hw, lat, ints, ids_out, xbc, cq, qfull, moe_a, moe_y, moe_w, moe_i};
         for (void* p : all)
             if (p)
                 (void) hipFree(p);
         x = x0 = o32 = logits = tap = y32 = nullptr;
         h1 = h2 = proj = q = ctx = act = hw = lat = nullptr;
         ints = ids_out = nullptr;
+        xbc = cq = qfull = moe_a = nullptr;
+        moe_y = moe_w = nullptr;
+        moe_i = nullptr;
     }
 };
 
@@ -279,6 +295,17 @@ int ensure_scratch(tllm_stack* s, int tokens, int want, int n_ints)
         HIP_OK(hipMalloc(&s->hw, W * wd * es));
         HIP_OK(hipMalloc((void**) &s->ints, NI * 4));
         HIP_OK(hipMalloc((void**) &s->ids_out, W * 4));
+        HIP_OK(hipMalloc(&s->xbc, T * std::max(s->max_conv, 1) * es));
+        HIP_OK(hipMalloc(&s->cq, T * std::max(s->max_qrank, 1) * es));
+        HIP_OK(hipMalloc(&s->qfull, T * std::max(s->max_qfull, 1) * es));
+        {
+            // a mixture of experts works on one row per (token, chosen expert)
+            const size_t pairs = T * (size_t) std::max(s->max_top, 1);
+            HIP_OK(hipMalloc(&s->moe_a, (s->max_top ? pairs * wd : 1) * es));
+            HIP_OK(hipMalloc((void**) &s->moe_y, (s->max_top ? pairs * wd : 1) * 4));
+            HIP_OK(hipMalloc((void**) &s->moe_w, pairs * 4));
+            HIP_OK(hipMalloc((void**) &s->moe_i, (3 * pairs + (size_t) s->max_experts + 1) * 4));
+        }
         HIP_OK(hipHostMalloc((void**) &s->pinned, NI * 4, hipHostMallocDefault));
         if (s->taps)
             HIP_OK(hipMalloc((void**) &s->tap, s->runs.size() * T * wd * 4));
@@ -375,25 +402,47 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.kind = MIX_HGRN2;
         else if (kind == "latent_attention")
             l.kind = MIX_LATENT;
+        else if (kind == "mamba2")
+            l.kind = MIX_MAMBA2;
         else
         {
-            set_error("tllm_stack_create: layer %d has mixer type '%s' (attention | latent_attention | hgrn2)", i, kind.c_str());
+            set_error("tllm_stack_create: layer %d has mixer type '%s' (attention | latent_attention | hgrn2 | mamba2)", i, kind.c_str());
             delete s;
             return nullptr;
         }
         l.heads = geti(s, p + "heads", 0);
-        l.dim = geti(s, p + "dim", 0);
+        l.dim = geti(s, p + (l.kind == MIX_MAMBA2 ? "state" : "dim"), 0);
         l.vdim = geti(s, p + "vdim", l.dim);
+        l.weights_of = geti(s, p + "weights_of", -1);
+        if (l.weights_of >= i || (l.weights_of >= 0 && s->layers[l.weights_of].weights_of >= 0))
+            return fail("weights_of names an earlier layer that has weights of its own");
         l.ff = geti(s, p + "ff", 0);
         if (l.heads < 1 || l.dim < 1 || l.vdim < 1 || l.ff < 0)
             return fail("a layer needs heads, dim and vdim");
         l.n_ctx = l.heads * l.vdim;
         const std::string mlp = gets(s, p + "mlp", "gelu_gate");
-        if (mlp != "gelu_gate" && mlp != "relu2")
-            return fail("a layer's mlp is gelu_gate or relu2");
-        l.mlp = mlp == "relu2" ? MLP_RELU2 : MLP_GELU_GATE;
-        if (l.mlp == MLP_RELU2 && !s->sequential)
-            return fail("the relu2 feed-forward is built for block=sequential");
+        if (mlp != "gelu_gate" && mlp != "relu2" && mlp != "moe")
+            return fail("a layer's mlp is gelu_gate, relu2 or moe");
+        l.mlp = mlp == "relu2" ? MLP_RELU2 : (mlp == "moe" ? MLP_MOE : MLP_GELU_GATE);
+        if (l.mlp != MLP_GELU_GATE && !s->sequential)
+            return fail("the relu2 and moe feed-forwards are built for block=sequential");
+        if ((l.kind == MIX_MAMBA2 || l.weights_of >= 0) && !s->sequential)
+            return fail("mamba2 layers and shared weights are built for block=sequential");
+        if (l.mlp == MLP_MOE && l.ff > 0)
+        {
+            l.experts = geti(s, p + "experts", 0);
+            l.identity = geti(s, p + "identity", 0);
+            l.top = geti(s, p + "top", 1);
+            l.route_groups = geti(s, p + "route_groups", 1);
+            l.route_keep = geti(s, p + "route_keep", l.route_groups);
+            l.route_scale = getd(s, p + "route_scale", 1.0);
+            const int ne = l.experts + l.identity;
+            if (l.experts < 1 || l.identity < 0 || ne > 1024 || l.top < 1 || l.top > 16 || l.top > ne || l.route_groups < 1 || ne % l.route_groups
+                || l.route_keep < 1 || l.route_keep > l.route_groups)
+                return fail("moe: experts >= 1, experts + identity <= 1024 in equal route_groups, 1 <= route_keep <= route_groups, top <= 16");
+            s->max_top = std::max(s->max_top, l.top);
+            s->max_experts = std::max(s->max_experts, l.experts);
+        }
         l.n_rg = s->hyper ? 0 : s->width;
         if (l.kind == MIX_LATENT)
         {
@@ -401,13 +450,31 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.rot_part = geti(s, p + "rot_dim", 0);
             l.rot_dims = geti(s, p + "rot_dims", l.rot_part);
             l.rot_base = getd(s, p + "rot_base", 10000);
+            l.rot_factor = getd(s, p + "rot_factor", 0);
+            l.rot_original = getd(s, p + "rot_original", 0);
+            l.rot_fast = getd(s, p + "rot_fast", 0);
+            l.rot_slow = getd(s, p + "rot_slow", 0);
             l.scale = getd(s, p + "scale", 1.0 / std::sqrt((double) (l.dim + l.rot_part)));
-            if (l.kv_rank < 1 || l.rot_part < 0 || l.rot_dims < 0 || (l.rot_dims & 1) || l.rot_dims > l.rot_part)
+            l.q_rank = geti(s, p + "q_rank", 0);
+            const std::string pairing = gets(s, p + "rot_pairing", "neighbours"), mk = gets(s, p + "mask", "causal");
+            if ((pairing != "neighbours" && pairing != "halves") || (mk != "causal" && mk != "window" && mk != "chunk"))
+                return fail("latent_attention: rot_pairing neighbours | halves, mask causal | window | chunk");
+            l.rot_halves = pairing == "halves";
+            l.mask = mk == "window" ? MASK_WINDOW : (mk == "chunk" ? MASK_CHUNK : MASK_CAUSAL);
+            l.mask_size = geti(s, p + "mask_size", 0);
+            l.sink = geti(s, p + "sink", 0);
+            if (l.kv_rank < 1 || l.rot_part < 0 || l.rot_dims < 0 || (l.rot_dims & 1) || l.rot_dims > l.rot_part || l.q_rank < 0)
                 return fail("latent_attention: kv_rank positive, rot_dims even and <= rot_dim");
+            if (l.mask != MASK_CAUSAL && l.mask_size < 1)
+                return fail("latent_attention: a window or chunk mask needs mask_size >= 1");
             l.kv_heads = 1;
-            l.n_q = l.heads * (l.dim + l.rot_part);
+            // columns of the mixer's projection: the queries of every head, or the query latent they are expanded from
+            l.n_q = l.q_rank > 0 ? l.q_rank : l.heads * (l.dim + l.rot_part);
             l.n_k = l.kv_rank + l.rot_part; // the down projection: latent | rotated key part
             l.n_v = 0;
+            s->max_qrank = std::max(s->max_qrank, l.q_rank);
+            if (l.q_rank > 0)
+                s->max_qfull = std::max(s->max_qfull, l.heads * (l.dim + l.rot_part));
             l.n_lat = l.heads * l.kv_rank;
             s->max_lat = std::max(s->max_lat, l.n_lat);
             s->max_q = std::max(s->max_q, l.heads * (l.kv_rank + l.rot_part));
@@ -452,6 +519,21 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.n_k = l.kv_heads * l.maps * l.dim;
             l.n_v = l.kv_heads * l.vdim;
         }
+        else if (l.kind == MIX_MAMBA2)
+        {
+            l.groups = geti(s, p + "groups", 1);
+            l.taps = geti(s, p + "conv", 4);
+            l.ssm_norm_groups = geti(s, p + "ssm_norm_groups", 1);
+            if (l.groups < 1 || l.heads % l.groups || l.ssm_norm_groups < 1 || (l.heads * l.vdim) % l.ssm_norm_groups
+                || !stack_ssm_serves(l.vdim, l.dim, l.taps))
+                return fail("mamba2: heads a multiple of groups, heads * vdim a multiple of ssm_norm_groups, conv 1 .. 16, state x vdim up to 32 x 1024");
+            // columns of the projection: z | x | B | C | dt; the convolution runs over x | B | C
+            l.n_conv = l.heads * l.vdim + 2 * l.groups * l.dim;
+            l.n_q = l.heads * l.vdim;
+            l.n_k = l.n_conv;
+            l.n_v = l.heads;
+            s->max_conv = std::max(s->max_conv, l.n_conv);
+        }
         else
         {
             if (!stack_hgrn2_serves(l.dim, l.vdim))
@@ -461,10 +543,11 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.n_v = l.heads * l.vdim;
         }
         l.n_mix = l.n_q + l.n_k + l.n_v + l.n_rg + l.n_gate;
-        s->max_proj = std::max(s->max_proj, std::max(l.n_mix, (l.mlp == MLP_RELU2 ? l.ff : 2 * l.ff) + l.n_rg));
+        const int ff_rows = l.mlp == MLP_MOE ? l.top : 1; // a mixture's products run on one row per (token, chosen expert)
+        s->max_proj = std::max(s->max_proj, std::max(l.n_mix, ff_rows * (l.mlp == MLP_RELU2 ? l.ff : 2 * l.ff) + l.n_rg));
         s->max_q = std::max(s->max_q, l.n_q);
         s->max_ctx = std::max(s->max_ctx, l.n_ctx);
-        s->max_ff = std::max(s->max_ff, l.ff);
+        s->max_ff = std::max(s->max_ff, ff_rows * l.ff);
     }
     // execution order
     auto add = [&](int layer, int pass, bool enters) {
@@ -569,6 +652,22 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
             const HostTensor* v = need(s, p + n, {len});
             return (!v || upload_f32(s, v->v.data(), v->v.size(), out)) ? -1 : 0;
         };
+        if (l.weights_of >= 0)
+        {
+            // the layer runs on another layer's weights: same description, same device tensors; caches and states go by run
+            const Layer& src = s->layers[(size_t) l.weights_of];
+            if (src.kind != l.kind || src.n_mix != l.n_mix || src.n_ctx != l.n_ctx || src.ff != l.ff || src.mlp != l.mlp || src.dim != l.dim
+                || src.heads != l.heads || src.experts != l.experts || src.identity != l.identity || src.kv_rank != l.kv_rank
+                || src.rot_part != l.rot_part || src.taps != l.taps)
+            {
+                set_error("tllm_stack_finalize: layer %d uses the weights of layer %d, but their shapes differ", (int) i, l.weights_of);
+                return -1;
+            }
+            const int from = l.weights_of;
+            l = src;
+            l.weights_of = from;
+            continue;
+        }
         if (norm_vec(p + "norm1", Wd, &l.norm1))
             return -1;
         const HostTensor* rg1 = nullptr;
@@ -598,13 +697,28 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
                     return -1;
             }
         }
-        const HostTensor* wq = need(s, p + "mix.q", {l.n_q, Wd});
-        const HostTensor* wk = need(s, p + (l.kind == MIX_ATTENTION ? "mix.k" : (l.kind == MIX_LATENT ? "mix.dkv" : "mix.f")), {l.n_k, Wd});
-        const HostTensor* wv = l.kind == MIX_LATENT ? nullptr : need(s, p + "mix.v", {l.n_v, Wd});
-        const HostTensor* wo = need(s, p + "mix.o", {Wd, l.n_ctx});
+        if (l.kind == MIX_MAMBA2)
+        {
+            const HostTensor* win = need(s, p + "mix.in", {l.n_mix, Wd});
+            const HostTensor* wo = need(s, p + "mix.o", {Wd, l.n_ctx});
+            const HostTensor* cw = need(s, p + "mix.conv", {l.n_conv, l.taps});
+            if (!win || !wo || !cw || upload_rows(s, {win}, &l.w_mix) || upload_rows(s, {wo}, &l.w_o)
+                || upload_f32(s, cw->v.data(), cw->v.size(), &l.conv_w) || vec("mix.conv.b", l.n_conv, &l.conv_b)
+                || vec("mix.dt_bias", l.heads, &l.dt_bias) || vec("mix.A_log", l.heads, &l.a_log) || vec("mix.D", l.heads, &l.d_skip)
+                || vec("mix.norm", l.n_ctx, &l.hnorm))
+                return -1;
+        }
+        const bool q_latent = l.kind == MIX_LATENT && l.q_rank > 0;
+        const HostTensor* wq = l.kind == MIX_MAMBA2 ? nullptr : need(s, p + (q_latent ? "mix.dq" : "mix.q"), {l.n_q, Wd});
+        const HostTensor* wk = l.kind == MIX_MAMBA2
+            ? nullptr
+            : need(s, p + (l.kind == MIX_ATTENTION ? "mix.k" : (l.kind == MIX_LATENT ? "mix.dkv" : "mix.f")), {l.n_k, Wd});
+        const HostTensor* wv = (l.kind == MIX_LATENT || l.kind == MIX_MAMBA2) ? nullptr : need(s, p + "mix.v", {l.n_v, Wd});
+        const HostTensor* wo = l.kind == MIX_MAMBA2 ? nullptr : need(s, p + "mix.o", {Wd, l.n_ctx});
         const HostTensor* wg = l.n_gate ? need(s, p + "mix.g", {l.n_gate, Wd}) : nullptr;
-        if (!wq || !wk || (!wv && l.kind != MIX_LATENT) || !wo || (l.n_gate && !wg))
+        if (l.kind != MIX_MAMBA2 && (!wq || !wk || (!wv && l.kind != MIX_LATENT) || !wo || (l.n_gate && !wg)))
             return -1;
+        if (l.kind != MIX_MAMBA2)
         {
             std::vector<const HostTensor*> rows = {wq, wk};
             if (wv)
@@ -629,6 +743,14 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
             const HostTensor* uk = need(s, p + "mix.uk", {H * D, C});
             const HostTensor* uv = need(s, p + "mix.uv", {H * E, C});
             if (!uk || !uv || norm_plain(p + "mix.dkv.norm", C, &l.lat_norm))
+                return -1;
+            if (q_latent)
+            {
+                const HostTensor* uq = need(s, p + "mix.uq", {H * (D + l.rot_part), l.q_rank});
+                if (!uq || upload_rows(s, {uq}, &l.w_uq) || norm_plain(p + "mix.dq.norm", l.q_rank, &l.cq_norm))
+                    return -1;
+            }
+            if (l.sink && vec("mix.sink", l.heads, &l.sinkv))
                 return -1;
             // W_uk^T per head, [kv_rank, dim]: the query side of the absorbed score is a product with these rows
             HostTensor tr;
@@ -686,12 +808,35 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
             if (l.weights == WEIGHTS_SIGMOID && vec("mix.pb", l.heads, &l.wbias))
                 return -1;
         }
-        else
+        else if (l.kind == MIX_HGRN2)
         {
             if (vec("mix.f.b", l.n_k, &l.f_bias) || vec("mix.lower", l.n_k, &l.lower) || vec("mix.norm", l.vdim, &l.hnorm))
                 return -1;
         }
-        if (l.ff > 0)
+        if (l.ff > 0 && l.mlp == MLP_MOE)
+        {
+            // experts stacked: [gate_e; up_e] rows per expert, then the down matrices; router and correction stay fp32
+            const int ne = l.experts + l.identity;
+            const HostTensor* rw = need(s, p + "mlp.router", {ne, Wd});
+            if (norm_vec(p + "norm2", Wd, &l.norm2) || !rw || upload_f32(s, rw->v.data(), rw->v.size(), &l.router_w))
+                return -1;
+            if (s->host.count(p + "mlp.correction") && vec("mlp.correction", ne, &l.correction))
+                return -1;
+            std::vector<const HostTensor*> gu, dn;
+            for (int e = 0; e < l.experts; ++e)
+            {
+                const std::string ep = p + "mlp.e" + std::to_string(e) + ".";
+                const HostTensor *g = need(s, ep + "gate", {l.ff, Wd}), *u = need(s, ep + "up", {l.ff, Wd}), *d = need(s, ep + "down", {Wd, l.ff});
+                if (!g || !u || !d)
+                    return -1;
+                gu.push_back(g);
+                gu.push_back(u);
+                dn.push_back(d);
+            }
+            if (upload_rows(s, gu, &l.w_gu) || upload_rows(s, dn, &l.w_down))
+                return -1;
+        }
+        else if (l.ff > 0)
         {
             if (norm_vec(p + "norm2", Wd, &l.norm2))
                 return -1;
@@ -745,6 +890,15 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
             if (alloc_zero(s, (size_t) s->blocks * l.kv_heads * l.maps * s->page * l.dim * s->es, &r.k_pool)
                 || alloc_zero(s, (size_t) s->blocks * l.kv_heads * s->page * l.vdim * s->es, &r.v_pool))
                 return -1;
+        }
+        else if (l.kind == MIX_MAMBA2)
+        {
+            void *st = nullptr, *cv = nullptr;
+            if (alloc_zero(s, (size_t) s->slots * l.heads * l.dim * l.vdim * 4, &st)
+                || alloc_zero(s, (size_t) s->slots * (l.taps - 1) * l.n_conv * 4, &cv))
+                return -1;
+            r.state = (float*) st;
+            r.conv_state = (float*) cv;
         }
         else
         {
@@ -880,6 +1034,40 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         g.ldc = l.n_mix;
         if (launch_stack_gemm(g, stream))
             return -1;
+        if (l.kind == MIX_MAMBA2)
+        {
+            StackSsmParams sp;
+            sp.dtype = s->dtype;
+            sp.tokens = T;
+            sp.entries = E;
+            sp.heads = l.heads;
+            sp.vdim = l.vdim;
+            sp.state = l.dim;
+            sp.groups = l.groups;
+            sp.taps = l.taps;
+            sp.proj = s->proj;
+            sp.ldp = l.n_mix;
+            sp.conv_w = l.conv_w;
+            sp.conv_b = l.conv_b;
+            sp.dt_bias = l.dt_bias;
+            sp.a_log = l.a_log;
+            sp.d_skip = l.d_skip;
+            sp.conv_state = r.conv_state;
+            sp.ssm_state = r.state;
+            sp.xbc = s->xbc;
+            sp.y32 = s->o32;
+            sp.tok_entry = d_tent;
+            sp.tok_pos = d_tpos;
+            sp.ent_slot = d_slot;
+            sp.ent_first = d_first;
+            sp.ent_count = d_count;
+            sp.ent_pos0 = d_pos0;
+            // convolution + silu (and the sequence's new tail), the recurrence with skip and gate, the norm in parts of the row
+            if (launch_stack_ssm_conv(sp, stream) || launch_stack_ssm_scan(sp, stream))
+                return -1;
+            return launch_stack_group_rmsnorm(s->ctx, nullptr, s->o32, nullptr, l.hnorm, nullptr, s->dtype, T, l.n_ctx, l.ssm_norm_groups, s->eps,
+                stream);
+        }
         if (l.kind == MIX_HGRN2)
         {
             StackHgrnParams hp;
@@ -938,16 +1126,43 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
             a.dim = C + R;
             a.vdim = C;
             a.rot_dims = l.rot_dims;
+            a.rot_halves = l.rot_halves;
+            a.mscale = l.mscale;
+            a.mask = l.mask;
+            a.mask_size = l.mask_size;
+            a.sink = l.sinkv;
             a.out = s->lat;
-            if (launch_stack_latent_prep(a, D, l.lat_norm, stream))
+            const void* q_src = s->proj;
+            int64_t ldq = l.n_mix;
+            if (l.q_rank > 0)
+            {
+                // queries through their own latent: norm of the first q_rank columns, then the expansion to every head's [plain | rotated]
+                if (launch_stack_row_rmsnorm(s->cq, l.q_rank, s->proj, l.n_mix, l.cq_norm, s->dtype, T, l.q_rank, s->eps, stream))
+                    return -1;
+                StackGemmParams uq;
+                uq.dtype = s->dtype;
+                uq.M = T;
+                uq.N = H * (D + R);
+                uq.K = l.q_rank;
+                uq.a = s->cq;
+                uq.lda = l.q_rank;
+                uq.w = l.w_uq;
+                uq.c = s->qfull;
+                uq.ldc = uq.N;
+                if (launch_stack_gemm(uq, stream))
+                    return -1;
+                q_src = s->qfull;
+                ldq = uq.N;
+            }
+            if (launch_stack_latent_prep(a, D, l.lat_norm, stream, q_src, ldq, l.n_q))
                 return -1;
             StackGemmParams qa;
             qa.dtype = s->dtype;
             qa.M = T;
             qa.N = C;
             qa.K = D;
-            qa.a = s->proj;
-            qa.lda = l.n_mix;
+            qa.a = q_src;
+            qa.lda = ldq;
             qa.w = l.w_ukT;
             qa.c = s->q;
             qa.ldc = (int64_t) H * (C + R);
@@ -1063,6 +1278,63 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
                 u.lda = Wd;
                 u.w = l.w_gu;
                 const void* act = s->act;
+                if (l.mlp == MLP_MOE)
+                {
+                    const size_t pairs = (size_t) T * l.top;
+                    StackMoeParams mp;
+                    mp.dtype = s->dtype;
+                    mp.tokens = T;
+                    mp.width = Wd;
+                    mp.experts = l.experts;
+                    mp.identity = l.identity;
+                    mp.top = l.top;
+                    mp.group_count = l.route_groups;
+                    mp.group_keep = l.route_keep;
+                    mp.scale = (float) l.route_scale;
+                    mp.h = s->h1;
+                    mp.router_w = l.router_w;
+                    mp.correction = l.correction;
+                    mp.topk_idx = s->moe_i;
+                    mp.slot_of_pair = s->moe_i + pairs;
+                    mp.pair_of_slot = s->moe_i + 2 * pairs;
+                    mp.group_off = s->moe_i + 3 * pairs;
+                    mp.topk_w = s->moe_w;
+                    mp.a_sorted = s->moe_a;
+                    if (launch_stack_moe_route(mp, stream) || launch_stack_moe_sort(mp, stream))
+                        return -1;
+                    // per expert: [gate; up] on its rows, silu(gate) * up, down in fp32; an expert's rows are at most one per token
+                    u.M = T;
+                    u.N = 2 * l.ff;
+                    u.a = s->moe_a;
+                    u.c = s->proj;
+                    u.ldc = u.N;
+                    u.batch = l.experts;
+                    u.stride_w = (int64_t) 2 * l.ff * Wd;
+                    u.group_off = mp.group_off;
+                    if (launch_stack_gemm(u, stream)
+                        || launch_stack_gelu_gate(s->act, s->proj, s->dtype, (int) pairs, l.ff, u.N, stream, GATE_SILU))
+                        return -1;
+                    StackGemmParams dn;
+                    dn.dtype = s->dtype;
+                    dn.out_f32 = 1;
+                    dn.M = T;
+                    dn.N = Wd;
+                    dn.K = l.ff;
+                    dn.a = s->act;
+                    dn.lda = l.ff;
+                    dn.w = l.w_down;
+                    dn.c = s->moe_y;
+                    dn.ldc = Wd;
+                    dn.batch = l.experts;
+                    dn.stride_w = (int64_t) Wd * l.ff;
+                    dn.group_off = mp.group_off;
+                    if (launch_stack_gemm(dn, stream) || launch_stack_moe_combine(mp, s->moe_y, s->y32, stream))
+                        return -1;
+                    pending = &l.hc[1];
+                    if (s->taps && hyper(nullptr, nullptr, nullptr, s->tap + ri * (size_t) T * Wd))
+                        return -1;
+                    continue;
+                }
                 if (l.mlp == MLP_RELU2)
                 {
                     u.N = l.ff;
@@ -1247,13 +1519,22 @@ int64_t tllm_stack_step_bytes(tllm_stack_t s, int32_t n_tokens, int64_t context_
     for (const Run& r : s->runs)
     {
         const Layer& l = s->layers[r.layer];
-        const int64_t ff_rows = l.ff > 0 ? (l.mlp == MLP_RELU2 ? 2 : 3) * (int64_t) l.ff + l.n_rg : 0;
+        int64_t ff_rows = l.ff > 0 ? (l.mlp == MLP_RELU2 ? 2 : 3) * (int64_t) l.ff + l.n_rg : 0;
+        if (l.ff > 0 && l.mlp == MLP_MOE)
+        {
+            // the experts that the step's tokens can reach at most, and the fp32 router
+            ff_rows *= std::min<int64_t>(l.experts, (int64_t) n_tokens * l.top);
+            bytes += (int64_t) (l.experts + l.identity) * s->width * 4;
+        }
         bytes += ((int64_t) l.n_mix + l.n_ctx + ff_rows) * s->width * s->es;
+        if (l.kind == MIX_LATENT && l.q_rank > 0)
+            bytes += (int64_t) l.heads * (l.dim + l.rot_part) * l.q_rank * s->es;
         if (l.kind == MIX_LATENT)
         {
             // the two per-head expansions, and per context token the key row [latent | rotated part] and the latent again as value
             bytes += (int64_t) l.heads * l.kv_rank * (l.dim + l.vdim) * s->es;
-            bytes += context_tokens * (2 * (int64_t) l.kv_rank + l.rot_part) * s->es;
+            const int64_t ctx = l.mask == MASK_CAUSAL ? context_tokens : std::min<int64_t>(context_tokens, (int64_t) n_entries * l.mask_size);
+            bytes += ctx * (2 * (int64_t) l.kv_rank + l.rot_part) * s->es;
         }
         else if (l.kind == MIX_ATTENTION)
         {
@@ -1261,6 +1542,8 @@ int64_t tllm_stack_step_bytes(tllm_stack_t s, int32_t n_tokens, int64_t context_
             const int64_t ctx = l.mask == MASK_CAUSAL ? context_tokens : std::min<int64_t>(context_tokens, (int64_t) n_entries * l.mask_size);
             bytes += ctx * ((int64_t) l.n_k + l.n_v) * s->es;
         }
+        else if (l.kind == MIX_MAMBA2)
+            bytes += 2 * (int64_t) n_entries * ((int64_t) l.heads * l.dim * l.vdim + (int64_t) (l.taps - 1) * l.n_conv) * 4;
         else
             bytes += 2 * (int64_t) n_entries * l.heads * l.dim * l.vdim * 4;
     }

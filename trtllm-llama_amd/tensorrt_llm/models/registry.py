@@ -6,12 +6,14 @@ import json
 import os
 
 from .llama.model import LLaMAForCausalLM
+from .rofozen.model import RofozenForCausalLM
 from .tolenex.model import TolenexForCausalLM
 from .vetipel.model import VetipelForCausalLM
 
 MODEL_REGISTRY = {
     'LlamaForCausalLM': LLaMAForCausalLM,
     'LLaMAForCausalLM': LLaMAForCausalLM,
+    'Rofozen': RofozenForCausalLM,
     'Tolenex': TolenexForCausalLM,
     'Vetipel': VetipelForCausalLM,
 }
