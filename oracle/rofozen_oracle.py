@@ -21,6 +21,28 @@ import math
 
 import numpy as np
 
+# A test may ask how much rounding of the activations moves a result: inside `with rounding(fn):` every projection's output, every
+# norm's output, the convolution's output, attention weights and the feed-forwards' hidden activations pass through fn (for
+# instance a rounding to bfloat16).  It is an estimate of a row's conditioning, not a model of any engine.
+_round = None
+
+
+class rounding(object):
+    def __init__(self, fn):
+        self.fn = fn
+
+    def __enter__(self):
+        global _round
+        self.old, _round = _round, self.fn
+
+    def __exit__(self, *exc):
+        global _round
+        _round = self.old
+
+
+def _r(x):
+    return x if _round is None else _round(x)
+
 
 def sigmoid(z):
     return 1.0 / (1.0 + np.exp(-z))
@@ -40,7 +62,7 @@ def gelu_tanh(z):
 
 def rms_norm(x, weight, eps):
     """x / sqrt(mean(x^2) + eps) * weight over the last axis."""
-    return x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps) * weight
+    return _r(x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps) * weight)
 
 
 def part_rms_norm(x, weight, parts, eps):
@@ -48,7 +70,7 @@ def part_rms_norm(x, weight, parts, eps):
     n, c = x.shape
     y = x.reshape(n, parts, c // parts)
     y = y / np.sqrt(np.mean(y * y, axis=-1, keepdims=True) + eps)
-    return y.reshape(n, c) * weight
+    return _r(y.reshape(n, c) * weight)
 
 
 # ------------------------------------------------------------------------------------------------ mamba2
@@ -80,9 +102,9 @@ def mamba2(h, w, p, m, eps):
     n = h.shape[0]
     H, P, N, G = m['heads'], m['vdim'], m['state'], m['groups']
     inner = H * P
-    proj = h @ w[p + 'in'].T
+    proj = _r(h @ w[p + 'in'].T)
     z, xbc, dt = proj[:, :inner], proj[:, inner:2 * inner + 2 * G * N], proj[:, 2 * inner + 2 * G * N:]
-    xbc = silu(causal_conv(xbc, w[p + 'conv'], w[p + 'conv.b']))
+    xbc = _r(silu(causal_conv(xbc, w[p + 'conv'], w[p + 'conv.b'])))
     x = xbc[:, :inner].reshape(n, H, P)
     b = xbc[:, inner:inner + G * N].reshape(n, G, N)
     c = xbc[:, inner + G * N:].reshape(n, G, N)
@@ -147,7 +169,7 @@ def sink_softmax(scores, vis, sink):
     den = e.sum(axis=-1, keepdims=True)
     if sink is not None:
         den = den + np.exp(sink - top)
-    return e / den
+    return _r(e / den)
 
 
 def latent_attention(h, w, p, m, eps, positions=None):
@@ -158,12 +180,12 @@ def latent_attention(h, w, p, m, eps, positions=None):
     rot = m.get('rot') or {}
     dims = int(rot.get('dims', 0))
     freq, mult = blended_frequencies(dims, float(rot.get('base', 10000.0)), rot.get('scaling')) if dims else (None, 1.0)
-    cq = rms_norm(h @ w[p + 'dq'].T, w[p + 'dq.norm'], eps)
-    q = (cq @ w[p + 'uq'].T).reshape(n, H, D + R)
-    q_plain, q_rot = q[..., :D], rotate_halves(q[..., D:], pos, dims, freq, mult)
-    dkv = h @ w[p + 'dkv'].T
+    cq = rms_norm(_r(h @ w[p + 'dq'].T), w[p + 'dq.norm'], eps)
+    q = _r(cq @ w[p + 'uq'].T).reshape(n, H, D + R)
+    q_plain, q_rot = q[..., :D], _r(rotate_halves(q[..., D:], pos, dims, freq, mult))
+    dkv = _r(h @ w[p + 'dkv'].T)
     c = rms_norm(dkv[:, :C], w[p + 'dkv.norm'], eps)
-    k_rot = rotate_halves(dkv[:, C:], pos, dims, freq, mult)           # one part for all heads
+    k_rot = _r(rotate_halves(dkv[:, C:], pos, dims, freq, mult))       # one part for all heads
     k_plain = (c @ w[p + 'uk'].T).reshape(n, H, D)
     v = (c @ w[p + 'uv'].T).reshape(n, H, E)
     vis = window_visible(n, int((m.get('mask') or {}).get('size', 0)))
@@ -171,13 +193,13 @@ def latent_attention(h, w, p, m, eps, positions=None):
     for a in range(H):
         s = (q_plain[:, a] @ k_plain[:, a].T + q_rot[:, a] @ k_rot.T) * m['scale']
         sink = float(w[p + 'sink'][a]) if (p + 'sink') in w else None
-        out[:, a] = sink_softmax(s, vis, sink) @ v[:, a]
+        out[:, a] = _r(sink_softmax(s, vis, sink) @ v[:, a])
     return out.reshape(n, H * E) @ w[p + 'o'].T
 
 
 # ------------------------------------------------------------------------------------------------ feed-forwards
 def dense_ff(h, w, p):
-    return (gelu_tanh(h @ w[p + 'gate'].T) * (h @ w[p + 'up'].T)) @ w[p + 'down'].T
+    return _r(_r(gelu_tanh(_r(h @ w[p + 'gate'].T))) * _r(h @ w[p + 'up'].T)) @ w[p + 'down'].T
 
 
 def route(h, w, p, r):
@@ -203,7 +225,7 @@ def route(h, w, p, r):
 
 
 def expert_ff(h, w, p):
-    return (silu(h @ w[p + 'gate'].T) * (h @ w[p + 'up'].T)) @ w[p + 'down'].T
+    return _r(_r(silu(_r(h @ w[p + 'gate'].T))) * _r(h @ w[p + 'up'].T)) @ w[p + 'down'].T
 
 
 def moe_ff(h, w, p, mlp):
@@ -248,3 +270,17 @@ def forward(tokens, w, cfg, return_layers=False):
         taps.append(x)
     logits = rms_norm(x, w['final.norm'], float(cfg['norm']['eps'])) @ w['head'].T
     return (logits, np.stack(taps)) if return_layers else logits
+
+
+def logits(tokens, w, cfg):
+    return forward(tokens, w, cfg)
+
+
+def greedy(prompt, w, cfg, n_new):
+    """The greedy continuation, recomputed from scratch for every token."""
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        nxt = int(np.argmax(forward(toks, w, cfg)[-1]))
+        out.append(nxt)
+        toks.append(nxt)
+    return out
