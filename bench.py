@@ -62,11 +62,13 @@ def parse():
     ap.add_argument('--parity-prompts', type=int, default=8, help='seeded prompts of the accuracy report')
     ap.add_argument('--cpu-tokens', type=int, default=0, help='CPU-baseline decode steps (0 = sized to ~20 s)')
     ap.add_argument('--cpu-threads', type=int, default=0)
-    ap.add_argument('--design', default='llama', choices=['llama', 'tolenex', 'vetipel'],
+    ap.add_argument('--design', default='llama', choices=['llama', 'tolenex', 'vetipel', 'rofozen'],
                     help="tolenex: a side report instead of the headline workload - prefill and decode throughput of the Tolenex design "
                          "(bfloat16, ragged stack engine) at layer sizes of real models, beside LLaMA fp16 at equal size; "
                          "vetipel: the same report for the Vetipel design, beside Tolenex (the closest model: same engine, bfloat16) and "
                          "LLaMA fp16 at equal size")
+    # (rofozen: the same report for the Rofozen design - mamba2 and latent-attention layers, dense and routed feed-forwards - beside
+    # Tolenex, the closest model: a recurrent / attention hybrid on the same engine in bfloat16, and Vetipel and LLaMA fp16 at equal size)
     ap.add_argument('--design-sizes', default='2048,4096', help='--design tolenex: comma list of model widths')
     ap.add_argument('--design-no-llama', action='store_true', help='--design tolenex: skip the LLaMA side (kernel traces of the new design alone)')
     ap.add_argument('--design-alone', action='store_true', help='--design vetipel: time that design only (kernel traces without its neighbours)')
@@ -605,6 +607,30 @@ def vetipel_config(width, layers, vocab=32000):
             'layers': [{'type': kinds[i % 4][0], 'mixer': dict(kinds[i % 4][1]), 'mlp': dict(ff)} for i in range(layers)]}
 
 
+def rofozen_config(width, layers, vocab=32000):
+    """A Rofozen configuration with the layer sizes of a LLaMA-like model of this width: mamba2 layers with heads of 64 channels over
+    128 state rows (inner size 2 x width, 8 groups, 4 taps), latent attention with a latent of 256 + 64 rotated dimensions under heads
+    of 64 + 64 query / key and 128 value dimensions behind a query latent of 3/8 width, windows of 512 tokens; the first layer's
+    feed-forward is dense (2.6875 x width), the others route 4 of 32 experts + 2 identities (2 groups, 1 kept) of a quarter of that
+    size.  Layers cycle mamba2 / mamba2 / latent / mamba2 on the second layer's weights."""
+    heads = width // 128
+    eff = -(-int(width * 2.6875 / 4) // 64) * 64
+    dense = {'kind': 'dense', 'ff': int(width * 2.6875)}
+    moe = {'kind': 'moe', 'expert': {'ff': eff},
+           'router': {'experts': 32, 'identity': 2, 'top': 4, 'scale': 2.5, 'groups': {'count': 2, 'keep': 1}}}
+    ssm = {'heads': 2 * width // 64, 'vdim': 64, 'state': 128, 'groups': 8, 'conv': 4, 'norm_groups': 8}
+    lat = {'heads': heads, 'dim': 64, 'rot_dim': 64, 'vdim': 128, 'kv_rank': 256, 'q_rank': width * 3 // 8, 'scale': 128 ** -0.5,
+           'mask': {'size': 512}, 'rot': {'dims': 64, 'base': 500000.0, 'scaling': {'factor': 4.0, 'original': 8192, 'fast': 32.0, 'slow': 1.0}}}
+    out = []
+    for i in range(layers):
+        k = i % 4
+        l = {'type': 'latent_attention' if k == 2 else 'mamba2', 'mixer': dict(lat if k == 2 else ssm), 'mlp': dict(dense if i == 0 else moe)}
+        if k == 3 and i >= 3:
+            l['weights_of'] = i - 2
+        out.append(l)
+    return {'architecture': 'Rofozen', 'vocab': vocab, 'width': width, 'norm': {'eps': 1e-6}, 'layers': out}
+
+
 def time_stack_model(torch, model, vocab, S, K, W, tag, row):
     """Prefill (one step of S prompt tokens) and decode (single tokens at context S, 1 and 4 sequences per step) of a stack-engine
     model in bfloat16 through RaggedGenerationSession.step; wall clock around synchronised calls."""
@@ -650,7 +676,15 @@ def tolenex_report(torch, args, dev):
         L = args.design_layers
         cfg = tolenex_config(width, L)
         row = dict(width=width, layers=L, context=S)
-        if args.design == 'vetipel':
+        if args.design == 'rofozen':
+            from tensorrt_llm.models import RofozenForCausalLM
+            rcfg = rofozen_config(width, L)
+            time_stack_model(torch, RofozenForCausalLM.from_random(rcfg, seed=1), rcfg['vocab'], S, K, W, 'rofozen', row)
+            if args.design_alone:
+                rows.append({k: (round(v, 3) if isinstance(v, float) else v) for k, v in row.items()})
+                print(f'[bench] {rows[-1]}', file=sys.stderr, flush=True)
+                continue
+        if args.design in ('vetipel', 'rofozen'):
             from tensorrt_llm.models import VetipelForCausalLM
             vcfg = vetipel_config(width, L)
             time_stack_model(torch, VetipelForCausalLM.from_random(vcfg, seed=1), vcfg['vocab'], S, K, W, 'vetipel', row)
@@ -735,7 +769,7 @@ def main():
         local = 0
     torch.cuda.set_device(local)
     dev = torch.device('cuda', local)
-    if args.design in ('tolenex', 'vetipel'):
+    if args.design in ('tolenex', 'vetipel', 'rofozen'):
         if world != 1:
             raise SystemExit(f'--design {args.design} is a one-GPU report')
         return tolenex_report(torch, args, dev)

@@ -271,6 +271,7 @@ struct StackMoeParams
     const void* h = nullptr;          // [tokens, width]
     const float* router_w = nullptr;  // [experts + identity, width]
     const float* correction = nullptr; // [experts + identity] or null
+    float* logits = nullptr;          // scratch [tokens, experts + identity]
     int32_t* topk_idx = nullptr;
     float* topk_w = nullptr;
     int32_t* group_off = nullptr;

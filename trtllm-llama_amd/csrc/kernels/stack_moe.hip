@@ -49,45 +49,94 @@ __device__ __forceinline__ void wave_argmax(float& v, int& idx)
     }
 }
 
-constexpr int RT = 4;         // tokens per workgroup: a router row is read once for all of them
+constexpr int RT = 8;         // tokens per logits workgroup: a router row is read once for all of them
 constexpr int MAX_OUT = 1024; // router outputs (experts + identities)
 constexpr int MAX_TOP = 16;
 
-// One workgroup of 4 waves per RT tokens.  The logits are fp32 dot products (a wave per router row, lanes over the width); wave w
-// then finishes token w: softmax, choice values, the kept groups, the top-k among them.
+// Router logits, fp32: workgroup (x, y) = 4 router rows (one per wave) x RT tokens; lanes split the width in float4 pieces where
+// rows are 16-byte aligned.  z [tokens, outputs].
 template <int DT>
-__global__ __launch_bounds__(256) void moe_route_kernel(const StackMoeParams p)
+__global__ __launch_bounds__(256) void moe_logits_kernel(const StackMoeParams p, float* z)
 {
-    extern __shared__ float sm[];
     const int NE = p.experts + p.identity, W = p.width;
-    float* z = sm;              // [RT][NE] logits, then scores
-    float* ch = z + RT * NE;    // [RT][NE] choice values
-    const int t0 = blockIdx.x * RT, lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
-    for (int e = wid; e < NE; e += 4)
-    {
-        float acc[RT];
+    const int e = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63, t0 = blockIdx.y * RT;
+    if (e >= NE)
+        return;
+    float acc[RT];
 #pragma unroll
-        for (int r = 0; r < RT; ++r)
-            acc[r] = 0.f;
-        const float* wr = p.router_w + (int64_t) e * W;
+    for (int r = 0; r < RT; ++r)
+        acc[r] = 0.f;
+    const float* wr = p.router_w + (int64_t) e * W;
+    const int nt = p.tokens - t0 < RT ? p.tokens - t0 : RT;
+    if ((W & 7) == 0)
+    {
+        for (int k = lane * 8; k < W; k += 64 * 8)
+        {
+            const float4 w0 = *reinterpret_cast<const float4*>(wr + k), w1 = *reinterpret_cast<const float4*>(wr + k + 4);
+            const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+            {
+                if (r < nt)
+                {
+                    float hv[8];
+                    if constexpr (DT == DT_BF16)
+                    {
+                        const uint4 u = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.h) + (int64_t) (t0 + r) * W + k);
+                        const uint32_t us[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                        {
+                            hv[2 * i] = __builtin_bit_cast(float, us[i] << 16);
+                            hv[2 * i + 1] = __builtin_bit_cast(float, us[i] & 0xffff0000u);
+                        }
+                    }
+                    else
+                    {
+                        const float* hp = reinterpret_cast<const float*>(p.h) + (int64_t) (t0 + r) * W + k;
+                        const float4 h0 = *reinterpret_cast<const float4*>(hp), h1 = *reinterpret_cast<const float4*>(hp + 4);
+                        hv[0] = h0.x, hv[1] = h0.y, hv[2] = h0.z, hv[3] = h0.w, hv[4] = h1.x, hv[5] = h1.y, hv[6] = h1.z, hv[7] = h1.w;
+                    }
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        acc[r] = fmaf(wv[i], hv[i], acc[r]);
+                }
+            }
+        }
+    }
+    else
+    {
         for (int k = lane; k < W; k += 64)
         {
             const float wv = wr[k];
 #pragma unroll
             for (int r = 0; r < RT; ++r)
-                if (t0 + r < p.tokens)
+                if (r < nt)
                     acc[r] = fmaf(wv, ld_el<DT>(p.h, (int64_t) (t0 + r) * W + k), acc[r]);
         }
-#pragma unroll
-        for (int r = 0; r < RT; ++r)
-        {
-            const float s = wave_sum(acc[r]);
-            if (lane == 0)
-                z[r * NE + e] = s;
-        }
     }
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+    {
+        const float sum = wave_sum(acc[r]);
+        if (lane == 0 && r < nt)
+            z[(int64_t) (t0 + r) * NE + e] = sum;
+    }
+}
+
+// One wave per token (4 per workgroup): softmax over the logits, choice values, the kept groups, the top-k among them.
+__global__ __launch_bounds__(256) void moe_select_kernel(const StackMoeParams p, const float* zg)
+{
+    extern __shared__ float sm[];
+    const int NE = p.experts + p.identity;
+    float* z = sm;              // [4][NE] scores
+    float* ch = z + 4 * NE;     // [4][NE] choice values
+    const int t0 = blockIdx.x * 4, lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    if (t0 + wid < p.tokens)
+        for (int e = lane; e < NE; e += 64)
+            z[wid * NE + e] = zg[(int64_t) (t0 + wid) * NE + e];
     __syncthreads();
-    const int t = t0 + wid; // RT == waves of the workgroup
+    const int t = t0 + wid;
     if (t >= p.tokens)
         return;
     float* zr = z + wid * NE;
@@ -308,13 +357,21 @@ int launch_stack_moe_route(const StackMoeParams& p, hipStream_t stream)
         return 0;
     if (!moe_ok(p, "stack_moe_route"))
         return -1;
-    const size_t lds = sizeof(float) * 2 * RT * (p.experts + p.identity);
-    const dim3 grid((p.tokens + RT - 1) / RT);
+    if (!p.logits)
+    {
+        set_error("stack_moe_route: no room for the logits");
+        return -1;
+    }
+    const int NE = p.experts + p.identity;
+    const dim3 lg((NE + 3) / 4, (p.tokens + RT - 1) / RT);
     if (p.dtype == DT_BF16)
-        hipLaunchKernelGGL((moe_route_kernel<DT_BF16>), grid, dim3(256), lds, stream, p);
+        hipLaunchKernelGGL((moe_logits_kernel<DT_BF16>), lg, dim3(256), 0, stream, p, p.logits);
     else
-        hipLaunchKernelGGL((moe_route_kernel<DT_FLOAT>), grid, dim3(256), lds, stream, p);
-    return launched("stack_moe_route");
+        hipLaunchKernelGGL((moe_logits_kernel<DT_FLOAT>), lg, dim3(256), 0, stream, p, p.logits);
+    if (launched("stack_moe_logits"))
+        return -1;
+    hipLaunchKernelGGL(moe_select_kernel, dim3((p.tokens + 3) / 4), dim3(256), sizeof(float) * 2 * 4 * NE, stream, p, p.logits);
+    return launched("stack_moe_select");
 }
 
 int launch_stack_moe_sort(const StackMoeParams& p, hipStream_t stream)

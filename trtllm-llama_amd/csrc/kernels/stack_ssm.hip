@@ -2,8 +2,11 @@
 // its per-sequence tail, and the recurrence over per-sequence state slots.  Step sizes, decays, the state and everything that
 // enters the recurrence are fp32 in both element types; `DT` is the storage type of the projection and of the convolution's output.
 #include "dev_utils.h"
+#include "launch_util.h"
 #include "stack_kernels.h"
 #include <algorithm>
+#include <cstdlib>
+#include <type_traits>
 
 namespace tllm
 {
@@ -190,6 +193,180 @@ __global__ __launch_bounds__(1024) void ssm_scan_kernel(const StackSsmParams p, 
     }
 }
 
+// The pipelined form of the same walk, for shapes whose chunk fits KMAX values per thread: the raw B, C, x, z and dt of chunk c + 1
+// are requested into registers before the recurrence of chunk c starts and land in the other half of a double-buffered LDS stage,
+// so a chunk waits for memory only at the start of an entry and has two barriers; step size and decay are computed once per row,
+// and the step size meets x (one product per thread and row) instead of every element of B.
+constexpr int KMAX = 8;
+
+template <int DT, int NSZ>
+__global__ __launch_bounds__(1024) void ssm_scan_pipe_kernel(const StackSsmParams p, int NS, int rc, int P)
+{
+    extern __shared__ float sm[];
+    // P: the columns of the head this workgroup keeps, [blockIdx.z P, + P) of its PH
+    const int PH = p.vdim, N = p.state, H = p.heads, G = p.groups, c0 = blockIdx.z * P;
+    const int inner = H * PH, GN = G * N, CH = inner + 2 * GN;
+    const int stage = rc * (2 + 2 * N + 2 * P);
+    float* os = sm + 2 * stage;      // [rc][NS][P]
+    const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, NT = blockDim.x;
+    const int g = h / (H / G);
+    const int s = tid / P, v = tid % P;
+    const bool live = s < NS && c0 + v < PH;
+    const int n0 = s * NSZ;
+    const int first = p.ent_first[e], count = p.ent_count[e];
+    float* sp = p.ssm_state + (((int64_t) p.ent_slot[e] * H + h) * N) * PH + c0 + v;
+    const bool carry = p.ent_pos0[e] > 0;
+    float S[NSZ];
+#pragma unroll
+    for (int j = 0; j < NSZ; ++j)
+        S[j] = (live && n0 + j < N && carry) ? sp[(int64_t) (n0 + j) * PH] : 0.f;
+    const float rate = -expf(p.a_log[h]), dtb = p.dt_bias[h], dsk = p.d_skip[h];
+    const bool vec4 = (N % NSZ) == 0 && (N & 3) == 0 && (P & 1) == 0; // (every LDS region then starts on 16 bytes)
+    // requested values stay raw bits until they are staged: a conversion next to its load would make the wave wait for it there
+    typedef typename std::conditional<DT == DT_BF16, uint16_t, float>::type Raw;
+    auto cvt = [](Raw r) -> float {
+        if constexpr (DT == DT_BF16)
+            return bf2f(r);
+        else
+            return r;
+    };
+    const Raw* xbc = reinterpret_cast<const Raw*>(p.xbc);
+    const Raw* prj = reinterpret_cast<const Raw*>(p.proj);
+    Raw rb[KMAX], rcv[KMAX], rx[KMAX], rz[KMAX], rdt = 0;
+    // element i = tid + k NT of a [rows, N] (or [rows, P]) chunk is (row, column) = (i / N, i % N): stepped, not divided, per k
+    const int qN = NT / N, mN = NT % N, qP = NT / P, mP = NT % P, rowN0 = tid / N, colN0 = tid % N;
+    const int kN = (rc * N + NT - 1) / NT, kP = (rc * P + NT - 1) / NT; // values per thread and chunk (<= KMAX)
+    auto request = [&](int t0) {
+        const int nt = count - t0 < rc ? count - t0 : rc;
+        int rowN = rowN0, colN = colN0, rowP = s, colP = v;
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+        {
+            // every lane loads from a row of the chunk (clamped), so that nothing branches around a load
+            if (k < kN)
+            {
+                const int64_t r = first + t0 + (rowN < nt ? rowN : nt - 1);
+                rb[k] = xbc[r * CH + inner + g * N + colN];
+                rcv[k] = xbc[r * CH + inner + GN + g * N + colN];
+            }
+            if (k < kP)
+            {
+                const int64_t r = first + t0 + (rowP < nt ? rowP : nt - 1);
+                const int col = c0 + colP < PH ? c0 + colP : PH - 1;
+                rx[k] = xbc[r * CH + h * PH + col];
+                rz[k] = prj[r * p.ldp + h * PH + col];
+            }
+            rowN += qN, colN += mN;
+            if (colN >= N)
+                colN -= N, ++rowN;
+            rowP += qP, colP += mP;
+            if (colP >= P)
+                colP -= P, ++rowP;
+        }
+        rdt = prj[(int64_t) (first + t0 + (tid < nt ? tid : nt - 1)) * p.ldp + 2 * inner + 2 * GN + h];
+    };
+    request(0);
+    int buf = 0;
+    for (int t0 = 0; t0 < count; t0 += rc, buf ^= 1)
+    {
+        const int nt = count - t0 < rc ? count - t0 : rc;
+        float* dd = sm + buf * stage;    // [rc][2] decay, step size
+        float* bs = dd + 2 * rc;         // [rc][N]
+        float* cs = bs + rc * N;         // [rc][N]
+        float* xs = cs + rc * N;         // [rc][P]
+        float* zs = xs + rc * P;         // [rc][P]
+#pragma unroll
+        for (int k = 0; k < KMAX; ++k)
+        {
+            const int i = tid + k * NT;
+            if (i < nt * N)
+            {
+                bs[i] = cvt(rb[k]);
+                cs[i] = cvt(rcv[k]);
+            }
+            if (i < nt * P)
+            {
+                xs[i] = cvt(rx[k]);
+                zs[i] = cvt(rz[k]);
+            }
+            if (i >= rc * N && i >= rc * P)
+                break;
+        }
+        if (tid < nt)
+        {
+            const float z = cvt(rdt) + dtb;
+            const float dt = z > 20.f ? z : log1pf(expf(z));
+            dd[2 * tid] = expf(rate * dt);
+            dd[2 * tid + 1] = dt;
+        }
+        __syncthreads();
+        if (t0 + rc < count)
+            request(t0 + rc); // in flight under this chunk's recurrence
+        if (live)
+        {
+            for (int tt = 0; tt < nt; ++tt)
+            {
+                const float a = dd[2 * tt], xd = xs[tt * P + v] * dd[2 * tt + 1];
+                const float* bt = bs + tt * N + n0;
+                const float* ct = cs + tt * N + n0;
+                float o = 0.f;
+                if (vec4)
+                {
+                    // rows of B and C are 16-byte aligned and the slice is whole: four values per LDS read
+#pragma unroll
+                    for (int j = 0; j < NSZ; j += 4)
+                    {
+                        const float4 b4 = *reinterpret_cast<const float4*>(bt + j), c4 = *reinterpret_cast<const float4*>(ct + j);
+                        S[j] = fmaf(a, S[j], b4.x * xd);
+                        S[j + 1] = fmaf(a, S[j + 1], b4.y * xd);
+                        S[j + 2] = fmaf(a, S[j + 2], b4.z * xd);
+                        S[j + 3] = fmaf(a, S[j + 3], b4.w * xd);
+                        o = fmaf(S[j], c4.x, o);
+                        o = fmaf(S[j + 1], c4.y, o);
+                        o = fmaf(S[j + 2], c4.z, o);
+                        o = fmaf(S[j + 3], c4.w, o);
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for (int j = 0; j < NSZ; ++j)
+                    {
+                        if (n0 + j < N)
+                        {
+                            S[j] = fmaf(a, S[j], bt[j] * xd);
+                            o = fmaf(S[j], ct[j], o);
+                        }
+                    }
+                }
+                os[(tt * NS + s) * P + v] = o;
+            }
+        }
+        __syncthreads();
+        for (int i = tid, tt = s, c = v; i < nt * P; i += NT)
+        {
+            float y = 0.f;
+            for (int s2 = 0; s2 < NS; ++s2)
+                y += os[(tt * NS + s2) * P + c];
+            y = fmaf(dsk, xs[i], y);
+            if (c0 + c < PH)
+                p.y32[(int64_t) (first + t0 + tt) * inner + h * PH + c0 + c] = y * silu_f(zs[i]);
+            tt += qP, c += mP;
+            if (c >= P)
+                c -= P, ++tt;
+        }
+        // (the next chunk stages into the other buffer; os is written again only behind the next chunk's first barrier, which no
+        // thread passes before it has finished these sums)
+    }
+    if (live)
+    {
+#pragma unroll
+        for (int j = 0; j < NSZ; ++j)
+            if (n0 + j < N)
+                sp[(int64_t) (n0 + j) * PH] = S[j];
+    }
+}
+
 // rows of state a thread keeps, for a head of P columns and N rows: the fewest that fit the workgroup, at least 4
 inline int slice_rows(int P, int N)
 {
@@ -245,10 +422,59 @@ int launch_stack_ssm_scan(const StackSsmParams& p, hipStream_t stream)
         return 0;
     if (!ssm_ok(p, "stack_ssm_scan"))
         return -1;
+    static const bool plain_only = [] {
+        const char* v = std::getenv("TLLM_STACK_SSM_PLAIN"); // measurement knob: 1 = every shape on the form without prefetch
+        return v && v[0] == '1';
+    }();
+    {
+        // The pipelined form.  A head's columns are cut over workgroups (halves, quarters, down to 16 columns) while the launch has
+        // fewer workgroups than the chip has CUs: a sequence's rows are walked in order, so the columns are what a long prompt of
+        // few sequences can spread.  Rows per chunk: as many as KMAX values per thread and 64 KiB of LDS hold.
+        const int cus = launch_util::device_cus();
+        int pc = p.vdim;
+        while (pc % 2 == 0 && pc / 2 >= 16 && (int64_t) p.entries * p.heads * (p.vdim / pc) < cus)
+            pc /= 2;
+        const int nsz = slice_rows(pc, p.state);
+        const int NS = nsz ? (p.state + nsz - 1) / nsz : 0;
+        const int threads = std::max(64, (NS * pc + 63) / 64 * 64);
+        int rc = 0;
+        for (int c : {16, 8, 4, 2})
+            if (nsz && c * p.state <= KMAX * threads && c * pc <= KMAX * threads && c <= threads
+                && sizeof(float) * (size_t) c * (2 * (2 + 2 * p.state + 2 * pc) + (size_t) NS * pc) <= 64 * 1024)
+            {
+                rc = c;
+                break;
+            }
+        if (rc > 0 && !plain_only)
+        {
+            const dim3 grid(p.entries, p.heads, p.vdim / pc);
+            const size_t plds = sizeof(float) * (size_t) rc * (2 * (2 + 2 * p.state + 2 * pc) + (size_t) NS * pc);
+#define TLLM_SSMP(DT, NSZ) hipLaunchKernelGGL((ssm_scan_pipe_kernel<DT, NSZ>), grid, dim3(threads), plds, stream, p, NS, rc, pc)
+#define TLLM_SSMP_DT(DT)                                                                                                                 \
+    switch (nsz)                                                                                                                          \
+    {                                                                                                                                     \
+    case 4: TLLM_SSMP(DT, 4); break;                                                                                                    \
+    case 8: TLLM_SSMP(DT, 8); break;                                                                                                    \
+    case 16: TLLM_SSMP(DT, 16); break;                                                                                                  \
+    default: TLLM_SSMP(DT, 32); break;                                                                                                  \
+    }
+            if (p.dtype == DT_BF16)
+            {
+                TLLM_SSMP_DT(DT_BF16)
+            }
+            else
+            {
+                TLLM_SSMP_DT(DT_FLOAT)
+            }
+#undef TLLM_SSMP_DT
+#undef TLLM_SSMP
+            return launched("stack_ssm_scan (pipelined)");
+        }
+    }
     const int nsz = slice_rows(p.vdim, p.state), NS = (p.state + nsz - 1) / nsz;
     const int threads = std::max(64, (NS * p.vdim + 63) / 64 * 64);
-    const size_t lds = sizeof(float) * ((size_t) RC * (1 + 2 * p.state + p.vdim + (size_t) NS * p.vdim));
     const dim3 grid(p.entries, p.heads);
+    const size_t lds = sizeof(float) * ((size_t) RC * (1 + 2 * p.state + p.vdim + (size_t) NS * p.vdim));
 #define TLLM_SSM(DT, NSZ) hipLaunchKernelGGL((ssm_scan_kernel<DT, NSZ>), grid, dim3(threads), lds, stream, p, NS)
 #define TLLM_SSM_DT(DT)                                                                                                                  \
     switch (nsz)                                                                                                                          \

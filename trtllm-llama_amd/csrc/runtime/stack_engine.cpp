@@ -129,7 +129,7 @@ struct tllm_stack
     void *xbc = nullptr, *cq = nullptr, *qfull = nullptr, *moe_a = nullptr;
     float *moe_y = nullptr, *moe_w = nullptr;
     int32_t* moe_i = nullptr;
-    int max_proj = 0, max_q = 0, max_ctx = 0, max_ff = 0, max_lat = 0, max_conv = 0, max_qrank = 0, max_qfull = 0, max_top = 0, max_experts = 0;
+    int max_proj = 0, max_q = 0, max_ctx = 0, max_ff = 0, max_lat = 0, max_conv = 0, max_qrank = 0, max_qfull = 0, max_top = 0, max_experts = 0, max_outputs = 0;
     int tap_tokens = 0;
 
     ~tllm_stack()
@@ -303,7 +303,7 @@ int ensure_scratch(tllm_stack* s, int tokens, int want, int n_ints)
             const size_t pairs = T * (size_t) std::max(s->max_top, 1);
             HIP_OK(hipMalloc(&s->moe_a, (s->max_top ? pairs * wd : 1) * es));
             HIP_OK(hipMalloc((void**) &s->moe_y, (s->max_top ? pairs * wd : 1) * 4));
-            HIP_OK(hipMalloc((void**) &s->moe_w, pairs * 4));
+            HIP_OK(hipMalloc((void**) &s->moe_w, (pairs + T * (size_t) (s->max_outputs + 1)) * 4));
             HIP_OK(hipMalloc((void**) &s->moe_i, (3 * pairs + (size_t) s->max_experts + 1) * 4));
         }
         HIP_OK(hipHostMalloc((void**) &s->pinned, NI * 4, hipHostMallocDefault));
@@ -442,6 +442,7 @@ tllm_stack_t tllm_stack_create(const char* config_text)
                 return fail("moe: experts >= 1, experts + identity <= 1024 in equal route_groups, 1 <= route_keep <= route_groups, top <= 16");
             s->max_top = std::max(s->max_top, l.top);
             s->max_experts = std::max(s->max_experts, l.experts);
+            s->max_outputs = std::max(s->max_outputs, ne);
         }
         l.n_rg = s->hyper ? 0 : s->width;
         if (l.kind == MIX_LATENT)
@@ -1299,6 +1300,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
                     mp.pair_of_slot = s->moe_i + 2 * pairs;
                     mp.group_off = s->moe_i + 3 * pairs;
                     mp.topk_w = s->moe_w;
+                    mp.logits = s->moe_w + pairs;
                     mp.a_sorted = s->moe_a;
                     if (launch_stack_moe_route(mp, stream) || launch_stack_moe_sort(mp, stream))
                         return -1;
