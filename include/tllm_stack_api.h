@@ -14,8 +14,13 @@
  * norm of the output; optionally projection biases, unit-RMS queries and keys, a per-head temperature, a linear or logarithmic
  * distance penalty, a sliding-window or chunked mask, sigmoid weights instead of a softmax, a softmax sink, a per-head output
  * gate), "latent_attention" (keys and values expanded from one low-rank latent per token plus one rotated key part shared by the
- * heads; the cache holds the latent and that part, attention runs in the absorbed form) and "hgrn2" (gated linear recurrence with
- * a lower-bounded forget gate, fp32 state).  Two block forms: parallel sublayers on one residual whose updates are gated by
+ * heads; the cache holds the latent and that part, attention runs in the absorbed form; optionally queries expanded from a normed
+ * latent of their own, half-split rotation pairs with YaRN-style frequency scaling, a window or chunk mask, a softmax sink), "hgrn2"
+ * (gated linear recurrence with a lower-bounded forget gate, fp32 state) and "mamba2" (selective state-space layer: a short causal
+ * convolution whose last inputs are part of the state, S <- exp(-exp(A_log) dt) S + dt B x^T per head over grouped B / C, skip, gate,
+ * RMS norm in parts of the row).  Feed-forwards: gated dense, relu^2, or a routed mixture of gated experts (softmax router with a
+ * choice correction, groups of experts of which only the best can be chosen, identity experts).  A layer may run on an earlier
+ * layer's weights (layer.<i>.weights_of), with a cache / state of its own.  Two block forms: parallel sublayers on one residual whose updates are gated by
  * sigmoid(W h + b), RMS norms in groups, a range of layers optionally run several times in a row (every pass with a cache / state
  * of its own); or sequential pre-norm sublayers on `streams` hyper-connected residual copies (u = sum_s in[s] x_s feeds the
  * sublayer, x_t <- sum_s mix[s, t] x_s + out[t] y lands its result; the output norm reads sum_s x_s).
@@ -42,17 +47,24 @@ typedef struct tllm_stack* tllm_stack_t;
  *   loop_start, loop_stop, loop_times (0, 0, 1: no loop), page_size (64), num_blocks, num_slots, debug_taps (0),
  *   block (parallel | sequential), residual (gated | hyper; parallel goes with gated, sequential with hyper), streams (1 .. 8),
  *   norm_offset (0: a norm weight is applied as norm_offset + stored value),
- *   per layer i: layer.<i>.type (attention | latent_attention | hgrn2), .heads, .dim, .vdim, .ff (0: no feed-forward),
- *     .mlp (gelu_gate: W_down (gelu_tanh(W_gate h) * W_up h) | relu2: W_down relu(W_up h)^2, sequential blocks only),
+ *   per layer i: layer.<i>.type (attention | latent_attention | hgrn2 | mamba2), .heads, .dim, .vdim, .ff (0: no feed-forward),
+ *     .weights_of (an earlier layer with weights of its own; sequential blocks only),
+ *     .mlp (gelu_gate: W_down (gelu_tanh(W_gate h) * W_up h) | relu2: W_down relu(W_up h)^2 | moe: .experts experts
+ *       W_down (silu(W_gate h) * W_up h) of size .ff plus .identity identity outputs, .top chosen per token among the .route_keep best
+ *       of .route_groups equal groups, weights = softmax score * .route_scale; relu2 and moe in sequential blocks only),
  *     attention: .kv_heads, .maps (1 | 2), .diff (the constant of the second map's weight and of the output scale 1 - diff),
  *       .scale, .softcap (0: none), .head_norm (0 | 1), .rot_dims, .rot_base, .rot_factor (0: no frequency scaling),
  *       .rot_original, .rot_fast, .rot_slow, .qkv_bias (0 | 1), .qk_norm (0 | 1: q and k / their RMS over dim), .head_temp (0 | 1),
  *       .pos_bias (none | linear: slope_h = 2^(-slope_base (h + 1) / heads) | log: r1_h ln(1 + r2_h (i - j))), .slope_base (8),
  *       .mask (causal | window | chunk), .mask_size, .weights (softmax | sigmoid), .sink (0 | 1), .out_gate (0 | 1);
- *     latent_attention: .kv_rank, .rot_dim (size of the shared rotated part), .rot_dims (how many of them turn), .rot_base, .scale.
+ *     latent_attention: .kv_rank, .rot_dim (size of the shared rotated part), .rot_dims (how many of them turn), .rot_base, .scale,
+ *       .q_rank (0: queries straight from the input), .rot_pairing (neighbours | halves), .rot_factor / .rot_original / .rot_fast /
+ *       .rot_slow, .mask, .mask_size, .sink;
+ *     mamba2: .state (rows of a head's state; takes the place of .dim), .groups, .conv (taps), .ssm_norm_groups.
  * Weights are named l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,lq1,lk1,lq2,lk2} (attention; with the options also q.b, k.b, v.b,
- * temp, r1, r2, sink, pb, g), l<i>.mix.{q,dkv,dkv.norm,uk,uv,o} (latent_attention), l<i>.mix.{q,f,f.b,lower,v,norm,o} (hgrn2),
- * l<i>.mlp.{gate,up,down}, l<i>.rg1, l<i>.rg1.b, l<i>.rg2, l<i>.rg2.b (gated residual), l<i>.hc{1,2}.{in,out,mix} (hyper
+ * temp, r1, r2, sink, pb, g), l<i>.mix.{q,dkv,dkv.norm,uk,uv,o} (latent_attention; with a query latent dq, dq.norm, uq instead of q;
+ * sink), l<i>.mix.{q,f,f.b,lower,v,norm,o} (hgrn2), l<i>.mix.{in,conv,conv.b,dt_bias,A_log,D,norm,o} (mamba2),
+ * l<i>.mlp.{gate,up,down} (moe: l<i>.mlp.e<k>.{gate,up,down}, l<i>.mlp.router, l<i>.mlp.correction), l<i>.rg1, l<i>.rg1.b, l<i>.rg2, l<i>.rg2.b (gated residual), l<i>.hc{1,2}.{in,out,mix} (hyper
  * residual; absent with one stream: the plain sum), embed, loop.step, final.norm, head; linear weights [out, in]. */
 tllm_stack_t tllm_stack_create(const char* config_text);
 

@@ -210,8 +210,10 @@ inline int launched(const char* what)
 
 // the lock-step tile shapes of the LDS-DMA kernel and what a tile of each kind costs per area (measured on fp16 operands; the
 // bfloat16 MFMA has the same rate and byte geometry): fewest workgroup rounds x area x cost
-int launch_glds_bf16(const GemmParams& g, hipStream_t stream)
+int launch_glds_bf16(const GemmParams& g, hipStream_t stream, int m_expected = 0)
 {
+    // m_expected: the rows a product of a grouped launch has on average (g.M is their bound, which sizes the grid): the tile shape is
+    // chosen for what is expected, or tall tiles would run half empty on every group
     struct Shape
     {
         int id, bm, bn;
@@ -223,7 +225,8 @@ int launch_glds_bf16(const GemmParams& g, hipStream_t stream)
     int pick = 0;
     for (const Shape& sh : shapes)
     {
-        const int64_t tiles = (int64_t) ((g.M + sh.bm - 1) / sh.bm) * ((g.N + sh.bn - 1) / sh.bn) * (g.batch > 1 ? g.batch : 1);
+        const int m = m_expected > 0 ? m_expected : g.M;
+        const int64_t tiles = (int64_t) ((m + sh.bm - 1) / sh.bm) * ((g.N + sh.bn - 1) / sh.bn) * (g.batch > 1 ? g.batch : 1);
         const double cost = (double) ((tiles + cus - 1) / cus) * sh.bm * sh.bn * sh.f;
         if (cost < best)
         {
@@ -315,7 +318,7 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream)
                 g.batch_w = p.stride_w * 2;
                 g.batch_c = p.stride_c * (p.out_f32 ? 4 : 2);
                 g.group_off = p.group_off;
-                rc = launch_glds_bf16(g, stream);
+                rc = launch_glds_bf16(g, stream, p.group_off ? p.group_rows : 0);
             }
             else
                 rc = launch_gemm_mfma(g, stream);

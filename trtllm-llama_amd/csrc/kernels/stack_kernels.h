@@ -53,6 +53,7 @@ struct StackGemmParams
     // Grouped form of a batch (a mixture of experts): device int32 [batch + 1]; product b takes rows [group_off[b], group_off[b + 1]) of
     // a and c (stride_a = stride_c = 0) and weight block b; M is the host's bound on the rows of one group.
     const int32_t* group_off = nullptr;
+    int32_t group_rows = 0; // the rows a group is expected to have (tile shapes are chosen for it), 0: M
 };
 int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream);
 

@@ -52,6 +52,7 @@ __device__ __forceinline__ void wave_argmax(float& v, int& idx)
 constexpr int RT = 8;         // tokens per logits workgroup: a router row is read once for all of them
 constexpr int MAX_OUT = 1024; // router outputs (experts + identities)
 constexpr int MAX_TOP = 16;
+constexpr int FEW_TOKENS = 8; // steps of this many tokens or fewer route in one launch and gather inside the sort
 
 // Router logits, fp32: workgroup (x, y) = 4 router rows (one per wave) x RT tokens; lanes split the width in float4 pieces where
 // rows are 16-byte aligned.  z [tokens, outputs].
@@ -124,23 +125,10 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const StackMoeParams p,
     }
 }
 
-// One wave per token (4 per workgroup): softmax over the logits, choice values, the kept groups, the top-k among them.
-__global__ __launch_bounds__(256) void moe_select_kernel(const StackMoeParams p, const float* zg)
+// One wave finishes one token: zr [outputs] holds its logits (LDS) and leaves as scores, cr [outputs] is room for the choice values.
+__device__ __forceinline__ void select_token(const StackMoeParams& p, float* zr, float* cr, int lane, int t)
 {
-    extern __shared__ float sm[];
     const int NE = p.experts + p.identity;
-    float* z = sm;              // [4][NE] scores
-    float* ch = z + 4 * NE;     // [4][NE] choice values
-    const int t0 = blockIdx.x * 4, lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
-    if (t0 + wid < p.tokens)
-        for (int e = lane; e < NE; e += 64)
-            z[wid * NE + e] = zg[(int64_t) (t0 + wid) * NE + e];
-    __syncthreads();
-    const int t = t0 + wid;
-    if (t >= p.tokens)
-        return;
-    float* zr = z + wid * NE;
-    float* cr = ch + wid * NE;
     float mx = -INFINITY;
     for (int e = lane; e < NE; e += 64)
         mx = fmaxf(mx, zr[e]);
@@ -232,9 +220,64 @@ __global__ __launch_bounds__(256) void moe_select_kernel(const StackMoeParams p,
     }
 }
 
+// One wave per token (4 per workgroup): softmax over the logits, choice values, the kept groups, the top-k among them.
+__global__ __launch_bounds__(256) void moe_select_kernel(const StackMoeParams p, const float* zg)
+{
+    extern __shared__ float sm[];
+    const int NE = p.experts + p.identity;
+    float* z = sm;              // [4][NE] scores
+    float* ch = z + 4 * NE;     // [4][NE] choice values
+    const int t0 = blockIdx.x * 4, lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    if (t0 + wid < p.tokens)
+        for (int e = lane; e < NE; e += 64)
+            z[wid * NE + e] = zg[(int64_t) (t0 + wid) * NE + e];
+    __syncthreads();
+    const int t = t0 + wid;
+    if (t >= p.tokens)
+        return;
+    select_token(p, z + wid * NE, ch + wid * NE, lane, t);
+}
+
+// Few tokens (a step of decoded tokens): one workgroup of 16 waves per token computes its logits (a wave per router row, 16-byte
+// pieces) and wave 0 finishes the token, in one launch.
+template <int DT>
+__global__ __launch_bounds__(1024) void moe_route_few_kernel(const StackMoeParams p)
+{
+    extern __shared__ float sm[];
+    const int NE = p.experts + p.identity, W = p.width, t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    for (int e = wid; e < NE; e += 16)
+    {
+        const float* wr = p.router_w + (int64_t) e * W;
+        float acc = 0.f;
+        if ((W & 7) == 0)
+        {
+            for (int k = lane * 8; k < W; k += 64 * 8)
+            {
+                const float4 w0 = *reinterpret_cast<const float4*>(wr + k), w1 = *reinterpret_cast<const float4*>(wr + k + 4);
+                const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    acc = fmaf(wv[i], ld_el<DT>(p.h, (int64_t) t * W + k + i), acc);
+            }
+        }
+        else
+        {
+            for (int k = lane; k < W; k += 64)
+                acc = fmaf(wr[k], ld_el<DT>(p.h, (int64_t) t * W + k), acc);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0)
+            sm[e] = acc;
+    }
+    __syncthreads();
+    if (wid == 0)
+        select_token(p, sm, sm + NE, lane, t);
+}
+
 // One workgroup: counts per expert, offsets, a slot per pair.  Which of an expert's slots a pair gets depends on the order of the
 // atomics; a row's product does not depend on its neighbours in a tile, so the results do not.
-__global__ __launch_bounds__(1024) void moe_sort_kernel(const StackMoeParams p)
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const StackMoeParams p, int gather_row_bytes)
 {
     extern __shared__ int si[];
     int* cnt = si;                  // [experts]
@@ -281,6 +324,25 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const StackMoeParams p)
             p.pair_of_slot[slot] = i;
         }
         p.slot_of_pair[i] = slot;
+    }
+    if (gather_row_bytes <= 0)
+        return;
+    // few pairs: the rows are copied here (a wave per pair) instead of by a launch of their own
+    __syncthreads();
+    const int lane = tid & 63;
+    for (int i = tid >> 6; i < pairs; i += NT >> 6)
+    {
+        const int slot = p.slot_of_pair[i];
+        if (slot < 0)
+            continue;
+        const char* src = reinterpret_cast<const char*>(p.h) + (int64_t) (i / p.top) * gather_row_bytes;
+        char* dst = reinterpret_cast<char*>(p.a_sorted) + (int64_t) slot * gather_row_bytes;
+        if ((gather_row_bytes & 15) == 0)
+            for (int b = lane * 16; b < gather_row_bytes; b += 64 * 16)
+                *reinterpret_cast<uint4*>(dst + b) = *reinterpret_cast<const uint4*>(src + b);
+        else
+            for (int b = lane * 2; b < gather_row_bytes; b += 64 * 2)
+                *reinterpret_cast<uint16_t*>(dst + b) = *reinterpret_cast<const uint16_t*>(src + b);
     }
 }
 
@@ -363,6 +425,14 @@ int launch_stack_moe_route(const StackMoeParams& p, hipStream_t stream)
         return -1;
     }
     const int NE = p.experts + p.identity;
+    if (p.tokens <= FEW_TOKENS)
+    {
+        if (p.dtype == DT_BF16)
+            hipLaunchKernelGGL((moe_route_few_kernel<DT_BF16>), dim3(p.tokens), dim3(1024), sizeof(float) * 2 * NE, stream, p);
+        else
+            hipLaunchKernelGGL((moe_route_few_kernel<DT_FLOAT>), dim3(p.tokens), dim3(1024), sizeof(float) * 2 * NE, stream, p);
+        return launched("stack_moe_route (few tokens)");
+    }
     const dim3 lg((NE + 3) / 4, (p.tokens + RT - 1) / RT);
     if (p.dtype == DT_BF16)
         hipLaunchKernelGGL((moe_logits_kernel<DT_BF16>), lg, dim3(256), 0, stream, p, p.logits);
@@ -381,10 +451,12 @@ int launch_stack_moe_sort(const StackMoeParams& p, hipStream_t stream)
     if (!moe_ok(p, "stack_moe_sort"))
         return -1;
     const size_t lds = sizeof(int) * (2 * (size_t) p.experts + 1);
-    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), lds, stream, p);
-    if (launched("stack_moe_sort"))
-        return -1;
     const int row_bytes = p.width * (p.dtype == DT_BF16 ? 2 : 4);
+    const bool few = p.tokens <= FEW_TOKENS;
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), lds, stream, p, few ? row_bytes : 0);
+    const int rc = launched("stack_moe_sort");
+    if (rc || few)
+        return rc;
     hipLaunchKernelGGL(moe_gather_kernel, dim3(p.tokens * p.top), dim3(256), 0, stream, p, row_bytes);
     return launched("stack_moe_gather");
 }

@@ -1313,6 +1313,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
                     u.batch = l.experts;
                     u.stride_w = (int64_t) 2 * l.ff * Wd;
                     u.group_off = mp.group_off;
+                    u.group_rows = (int) std::min<int64_t>(T, (pairs + l.experts - 1) / l.experts);
                     if (launch_stack_gemm(u, stream)
                         || launch_stack_gelu_gate(s->act, s->proj, s->dtype, (int) pairs, l.ff, u.N, stream, GATE_SILU))
                         return -1;
@@ -1330,6 +1331,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
                     dn.batch = l.experts;
                     dn.stride_w = (int64_t) Wd * l.ff;
                     dn.group_off = mp.group_off;
+                    dn.group_rows = u.group_rows;
                     if (launch_stack_gemm(dn, stream) || launch_stack_moe_combine(mp, s->moe_y, s->y32, stream))
                         return -1;
                     pending = &l.hc[1];
