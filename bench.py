@@ -647,13 +647,13 @@ def time_stack_model(torch, model, vocab, S, K, W, tag, row):
     row[f'{tag}_prefill_tokens_per_s'] = S / t_prefill
     for batch in (1, 4):
         ids = ['p'] + [f'q{b}' for b in range(1, batch)]
-        for rid in ids[1:]:
-            sess.step([(rid, prompt, [])])
+        for b, rid in enumerate(ids[1:]):  # every sequence its own tokens (a router would send equal tokens to equal experts)
+            sess.step([(rid, np.random.default_rng(b + 1).integers(0, vocab, S).tolist(), [])])
         for _ in range(W):
-            sess.step([(rid, [7], [0]) for rid in ids], return_logits=False)
+            sess.step([(rid, [7 + b], [0]) for b, rid in enumerate(ids)], return_logits=False)
         t0 = time.perf_counter()
         for _ in range(K):
-            sess.step([(rid, [7], [0]) for rid in ids], return_logits=False)
+            sess.step([(rid, [7 + b], [0]) for b, rid in enumerate(ids)], return_logits=False)
         dt = time.perf_counter() - t0
         row[f'{tag}_decode_b{batch}_tokens_per_s'] = batch * K / dt
         row[f'{tag}_decode_b{batch}_ms_per_step'] = dt * 1e3 / K

@@ -115,6 +115,9 @@ __global__ __launch_bounds__(64 * (WM * WN * KG + LW)) void gemm_glds_kernel(con
     // contiguous range of tiles so that the tiles sharing an A row-panel / W column-panel share an L2
     const int nwg = gridDim.x;
     int wg = blockIdx.x;
+    // (a grouped product has fewer tiles than the grid, the first ids: in launch order they already go round the XCDs, while
+    // contiguous ranges per XCD would leave every group's tiles on the first XCDs)
+    if (!(WT == W_BF16 && p.group_off))
     {
         const int q = nwg >> 3, r = nwg & 7, xcd = wg & 7, idx = wg >> 3;
         wg = (xcd < r ? xcd * (q + 1) : r * (q + 1) + (xcd - r) * q) + idx;
