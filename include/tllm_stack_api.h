@@ -98,7 +98,8 @@ int32_t tllm_stack_num_slots(tllm_stack_t s);
 int32_t tllm_stack_vocab(tllm_stack_t s);
 int32_t tllm_stack_layer_runs(tllm_stack_t s); /* layers as executed, a looped layer counted once per pass */
 int64_t tllm_stack_weight_bytes(tllm_stack_t s);
-/* bytes one step moves at least: weights once, plus the cache / state the given contexts touch (roofline denominators) */
+/* bytes one step moves at least: weights once, plus the cache / state the given contexts touch (roofline denominators); of a
+ * routed feed-forward the experts that the step's tokens reach when every choice falls on another expert */
 int64_t tllm_stack_step_bytes(tllm_stack_t s, int32_t n_tokens, int64_t context_tokens, int32_t n_entries);
 
 /* debug_taps=1: the residual stream behind layer run `run` of the last step (the sum of the streams, if there are several), fp32

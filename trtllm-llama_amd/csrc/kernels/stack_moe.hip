@@ -256,9 +256,27 @@ __global__ __launch_bounds__(1024) void moe_route_few_kernel(const StackMoeParam
             {
                 const float4 w0 = *reinterpret_cast<const float4*>(wr + k), w1 = *reinterpret_cast<const float4*>(wr + k + 4);
                 const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+                float hv[8];
+                if constexpr (DT == DT_BF16)
+                {
+                    const uint4 u = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.h) + (int64_t) t * W + k);
+                    const uint32_t us[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        hv[2 * i] = __builtin_bit_cast(float, us[i] << 16);
+                        hv[2 * i + 1] = __builtin_bit_cast(float, us[i] & 0xffff0000u);
+                    }
+                }
+                else
+                {
+                    const float* hp = reinterpret_cast<const float*>(p.h) + (int64_t) t * W + k;
+                    const float4 h0 = *reinterpret_cast<const float4*>(hp), h1 = *reinterpret_cast<const float4*>(hp + 4);
+                    hv[0] = h0.x, hv[1] = h0.y, hv[2] = h0.z, hv[3] = h0.w, hv[4] = h1.x, hv[5] = h1.y, hv[6] = h1.z, hv[7] = h1.w;
+                }
 #pragma unroll
                 for (int i = 0; i < 8; ++i)
-                    acc = fmaf(wv[i], ld_el<DT>(p.h, (int64_t) t * W + k + i), acc);
+                    acc = fmaf(wv[i], hv[i], acc);
             }
         }
         else
