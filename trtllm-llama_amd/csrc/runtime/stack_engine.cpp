@@ -13,6 +13,12 @@
 //   P1 = h1 [Wq; Wk; Wv; Wg]^T  (latent attention: [Wq; Wdkv])    mixer as above, per-head output gate inside the attention launch
 //   y = ctx Wo^T (fp32);  x_t <- sum_s mix1[s, t] x_s + out1[t] y   folded into the next launch that reads the streams
 //   h2 = norm2(sum_s in2[s] x_s);  a = relu(h2 Wup^T)^2 (product epilogue);  y = a Wdown^T;  x_t <- sum_s mix2[s, t] x_s + out2[t] y
+// A mamba2 mixer is  P1 = h1 W_in^T = [z | x | B | C | dt]  ->  convolution + silu of x | B | C (and the sequence's new tail)  ->  the
+// recurrence with skip and gate  ->  RMS norm in parts of the row;  a latent layer with a query latent projects [W_dq; W_dkv], norms
+// the query latent and expands it before the latent's pointwise part.  A routed feed-forward is  router (fp32 logits, softmax, kept
+// groups, top-k)  ->  (token, expert) pairs ordered by expert  ->  [gate_e; up_e] grouped product  ->  silu(gate) * up  ->  down_e
+// grouped product in fp32  ->  weighted sum per token (identity experts add w h).  A layer with weights_of runs on another layer's
+// device tensors; caches and states belong to runs.
 // The residual streams are fp32 in both element types.
 #include "../../../include/tllm_stack_api.h"
 #include "../kernels/stack_kernels.h"
