@@ -198,6 +198,7 @@ __global__ __launch_bounds__(1024) void ssm_scan_kernel(const StackSsmParams p, 
 // so a chunk waits for memory only at the start of an entry and has two barriers; step size and decay are computed once per row,
 // and the step size meets x (one product per thread and row) instead of every element of B.
 constexpr int KMAX = 8;
+constexpr size_t kMaxLds = 128 * 1024; // of a CU's 160 KiB
 
 template <int DT, int NSZ>
 __global__ __launch_bounds__(1024) void ssm_scan_pipe_kernel(const StackSsmParams p, int NS, int rc, int P)
@@ -429,7 +430,7 @@ int launch_stack_ssm_scan(const StackSsmParams& p, hipStream_t stream)
     {
         // The pipelined form.  A head's columns are cut over workgroups (halves, quarters, down to 16 columns) while the launch has
         // fewer workgroups than the chip has CUs: a sequence's rows are walked in order, so the columns are what a long prompt of
-        // few sequences can spread.  Rows per chunk: as many as KMAX values per thread and 64 KiB of LDS hold.
+        // few sequences can spread.  Rows per chunk: as many as KMAX values per thread and 128 KiB of LDS hold.
         const int cus = launch_util::device_cus();
         int pc = p.vdim;
         while (pc % 2 == 0 && pc / 2 >= 16 && (int64_t) p.entries * p.heads * (p.vdim / pc) < cus)
@@ -440,7 +441,7 @@ int launch_stack_ssm_scan(const StackSsmParams& p, hipStream_t stream)
         int rc = 0;
         for (int c : {16, 8, 4, 2})
             if (nsz && c * p.state <= KMAX * threads && c * pc <= KMAX * threads && c <= threads
-                && sizeof(float) * (size_t) c * (2 * (2 + 2 * p.state + 2 * pc) + (size_t) NS * pc) <= 64 * 1024)
+                && sizeof(float) * (size_t) c * (2 * (2 + 2 * p.state + 2 * pc) + (size_t) NS * pc) <= kMaxLds)
             {
                 rc = c;
                 break;
@@ -449,7 +450,12 @@ int launch_stack_ssm_scan(const StackSsmParams& p, hipStream_t stream)
         {
             const dim3 grid(p.entries, p.heads, p.vdim / pc);
             const size_t plds = sizeof(float) * (size_t) rc * (2 * (2 + 2 * p.state + 2 * pc) + (size_t) NS * pc);
-#define TLLM_SSMP(DT, NSZ) hipLaunchKernelGGL((ssm_scan_pipe_kernel<DT, NSZ>), grid, dim3(threads), plds, stream, p, NS, rc, pc)
+#define TLLM_SSMP(DT, NSZ)                                                                                                               \
+    do                                                                                                                                    \
+    {                                                                                                                                     \
+        launch_util::ensure_dynamic_lds(reinterpret_cast<const void*>(&ssm_scan_pipe_kernel<DT, NSZ>), plds > 64 * 1024 ? kMaxLds : 0);   \
+        hipLaunchKernelGGL((ssm_scan_pipe_kernel<DT, NSZ>), grid, dim3(threads), plds, stream, p, NS, rc, pc);                            \
+    } while (0)
 #define TLLM_SSMP_DT(DT)                                                                                                                 \
     switch (nsz)                                                                                                                          \
     {                                                                                                                                     \
