@@ -964,6 +964,9 @@ bool stack_attention_tiled(const StackAttnParams& p)
 {
     const bool std_shape = (p.dim == 32 || p.dim == 64 || p.dim == 128) && (p.vdim == 32 || p.vdim == 64 || p.vdim == 128);
     const bool latent_shape = p.maps == 1 && p.kv_heads == 1 && ((p.dim == 160 && p.vdim == 128) || (p.dim == 320 && p.vdim == 256));
+    // what only the general kernels do: head-mixed weights, a gate per channel, kept first keys under a window
+    if (p.talk || (p.out_gate && p.gate_wide) || p.mask_keep > 0)
+        return false;
     return p.dtype == DT_BF16 && (std_shape || latent_shape) && p.page % 32 == 0 && p.max_count > 0 && p.entries > 0 && !(reinterpret_cast<uintptr_t>(p.q) & 15)
         && !(reinterpret_cast<uintptr_t>(p.k_pool) & 15) && !(reinterpret_cast<uintptr_t>(p.v_pool) & 7);
 }

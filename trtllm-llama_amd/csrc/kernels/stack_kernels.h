@@ -64,6 +64,29 @@ int launch_stack_gemm(const StackGemmParams& p, hipStream_t stream);
 // written to x + c * copy_stride, c < copies (residual streams that all start from the embedding output)
 int launch_stack_embed(float* x, float* keep, const int32_t* ids, const void* table, int32_t dtype, int32_t tokens, int32_t width,
     int32_t vocab, float scale, hipStream_t stream, int32_t copies = 1, int64_t copy_stride = 0);
+// A hashed pair embedding on top of the rows above: x[t, :] += pair_table[row(t), :], row = (prev[t] * mul_prev + ids[t] * mul_cur) mod
+// buckets (64-bit arithmetic), or the extra row `buckets` where prev[t] < 0 (a sequence's first token).  pair_table [buckets + 1, width].
+int launch_stack_pair_embed(float* x, const int32_t* ids, const int32_t* prev, const void* pair_table, int32_t dtype, int32_t tokens,
+    int32_t width, int32_t buckets, int32_t mul_prev, int32_t mul_cur, hipStream_t stream, int32_t copies = 1, int64_t copy_stride = 0);
+// Token shift: h[t, :] = n[t, :] + (n[t - 1, :] - n[t, :]) * mu[:] over fp32 rows n (a norm's output), t - 1 the previous token of the
+// same sequence: the row above inside an entry, for an entry's first row the sequence's carried row carry[slot, :] (zeros when the
+// entry starts its sequence).  The carry then takes the entry's last row of n.  h in the element type; n is not changed.
+struct StackShiftParams
+{
+    int32_t dtype = DT_BF16;
+    int32_t tokens = 0, entries = 0, width = 0;
+    const float* n = nullptr;  // [tokens, width]
+    const float* mu = nullptr; // [width]
+    float* carry = nullptr;    // [slots, width]
+    void* h = nullptr;         // [tokens, width]
+    const int32_t* tok_entry = nullptr;
+    const int32_t* tok_pos = nullptr;
+    const int32_t* ent_slot = nullptr;
+    const int32_t* ent_first = nullptr;
+    const int32_t* ent_count = nullptr;
+    const int32_t* ent_pos0 = nullptr;
+};
+int launch_stack_token_shift(const StackShiftParams& p, hipStream_t stream);
 // x[t, :] += (add ? add[t, :] : 0) + (row ? row[:] : 0): the entry of a pass over a looped layer range
 int launch_stack_pass_entry(float* x, const float* add, const float* row, int32_t tokens, int32_t width, hipStream_t stream);
 // RMS norm in `groups` equal consecutive parts of the row, every part divided by its own sqrt(mean(part^2) + eps); the two
@@ -93,6 +116,7 @@ struct StackHyperParams
     const float* w = nullptr;   // [width] norm weight as applied (any offset already added)
     float eps = 1e-5f;
     float* sum_out = nullptr;
+    float* h32 = nullptr;          // [tokens, width] or null: the normed row in fp32 as well (a token shift reads it)
     const int32_t* rows = nullptr; // [tokens] or null
 };
 int launch_stack_hyper_norm(const StackHyperParams& p, hipStream_t stream);
@@ -130,16 +154,27 @@ struct StackAttnParams
     const float* slope = nullptr;
     const float* log_r1 = nullptr;
     const float* log_r2 = nullptr;
-    // mask: which keys j <= i a row sees.  MASK_WINDOW: i - j < mask_size; MASK_CHUNK: floor(i / mask_size) == floor(j / mask_size)
-    int32_t mask = 0, mask_size = 0;
+    // mask: which keys j <= i a row sees.  MASK_WINDOW: i - j < mask_size; MASK_CHUNK: floor(i / mask_size) == floor(j / mask_size);
+    // mask_keep > 0 (windows): the sequence's first mask_keep keys stay visible to every later row, at their true positions
+    int32_t mask = 0, mask_size = 0, mask_keep = 0;
     // weights: WEIGHTS_SOFTMAX, its denominator also holding exp(sink[h]) when sink is set (a logit without key or value);
     // WEIGHTS_SIGMOID: weight = sigmoid(score + wbias[h]) per key, not normalised over keys
     int32_t weights = 0;
     const float* sink = nullptr;
     const float* wbias = nullptr;
-    // the head's output times sigmoid(out_gate[t * ld_gate + h]) (pre-activations in the element type), null = none
+    // the head's output times sigmoid(out_gate[t * ld_gate + h]) (pre-activations in the element type), null = none;
+    // gate_wide: one gate per output channel, out_gate[t * ld_gate + h * vdim + c]
     const void* out_gate = nullptr;
     int64_t ld_gate = 0;
+    int32_t gate_wide = 0;
+    // talking heads: talk [heads, heads] fp32 on the device, null = none.  After the softmax (sink included in the denominators) head
+    // h's weight on key j becomes sum_g talk[h * heads + g] w_g(i, j); head h applies it to the values of its own key/value head.
+    const float* talk = nullptr;
+    // values_are_keys: the layer has no value projection; a token's value row is its key as projected (unrotated, unnormed); vdim == dim
+    int32_t values_are_keys = 0;
+    // weights of the q / k norm (qk_unit_norm), fp32 [dim] each, null = plain unit RMS
+    const float* q_norm_w = nullptr;
+    const float* k_norm_w = nullptr;
     // the projection's rows before anything else: + bias (fp32 [q | k | v columns]), then q and k of every head and map divided by
     // their root mean square over dim (qk_unit_norm, eps)
     const float* bias = nullptr;
@@ -170,6 +205,9 @@ int launch_stack_attention(const StackAttnParams& p, hipStream_t stream);
 size_t stack_attn_workspace_floats(int32_t heads, int32_t maps, int32_t vdim); // floats of split_ws a layer of this shape needs
 // frequencies of the rotation with YaRN-style scaling (factor <= 0: none): fills freq[dims / 2], returns the cos / sin multiplier
 float stack_rope_freqs(float* freq, int32_t dims, double base, double factor, double original, double fast, double slow);
+// frequencies with the three-band scaling by wavelength l = 2 pi / f: f stays where l < original / high, becomes f / factor where
+// l > original / low, and is blended by s = (original / l - low) / (high - low) between (factor <= 0: none)
+void stack_rope_freqs_banded(float* freq, int32_t dims, double base, double factor, double original, double low, double high);
 
 // ---------------------------------------------------------------------------------------------
 // Latent attention: a token leaves one latent c [rank] (RMS-normed with a plain weight) and one rotated key part [rot] that all
@@ -242,6 +280,10 @@ struct StackSsmParams
     float* ssm_state = nullptr;     // [slots, heads, state, vdim]
     void* xbc = nullptr;            // scratch [tokens, channels], element type
     float* y32 = nullptr;           // [tokens, inner]
+    // launch_stack_ssm_conv alone, for another layer kind: conv_channels > 0 channels that start at column conv_col of proj
+    // (instead of the x | B | C columns behind z); conv_b may be null
+    int32_t conv_channels = 0;
+    int64_t conv_col = 0;
     const int32_t* tok_entry = nullptr;
     const int32_t* tok_pos = nullptr;
     const int32_t* ent_slot = nullptr;
@@ -269,6 +311,8 @@ struct StackMoeParams
     int32_t tokens = 0, width = 0;
     int32_t experts = 0, identity = 0, top = 0, group_count = 1, group_keep = 1;
     float scale = 1.f;
+    int32_t score = 0;        // ROUTE_SOFTMAX: s = softmax(z) over all outputs; ROUTE_SIGMOID: s = sigmoid(z), every output by itself
+    int32_t weight_input = 0; // 1: the weight multiplies the expert's input row (a_sorted = w h), the outputs are summed unweighted
     const void* h = nullptr;          // [tokens, width]
     const float* router_w = nullptr;  // [experts + identity, width]
     const float* correction = nullptr; // [experts + identity] or null
@@ -280,9 +324,48 @@ struct StackMoeParams
     int32_t* pair_of_slot = nullptr;  // [tokens * top], -1 behind the last used slot
     void* a_sorted = nullptr;         // [tokens * top, width]
 };
+constexpr int32_t ROUTE_SOFTMAX = 0, ROUTE_SIGMOID = 1;
 int launch_stack_moe_route(const StackMoeParams& p, hipStream_t stream);
 int launch_stack_moe_sort(const StackMoeParams& p, hipStream_t stream);
 int launch_stack_moe_combine(const StackMoeParams& p, const float* y_sorted, float* y, hipStream_t stream);
+
+// ---------------------------------------------------------------------------------------------
+// Gated delta rule with one decay per key channel.  Per head h a state S [dim, vdim] (fp32, one per slot); head h reads the q / k
+// head h / (heads / qk_heads).  x [tokens, channels] holds q (qk_heads * dim) | k (qk_heads * dim) | v (heads * vdim) behind their
+// convolution and silu.  Per token, in fp32:
+//   q <- q / sqrt(sum q^2 + 1e-6) / sqrt(dim),  k <- k / sqrt(sum k^2 + 1e-6),  beta = sigmoid(beta_raw[t, h]),
+//   g[d] = exp(-exp(a_log[h]) * softplus(decay_raw[t, h * dim + d] + dt_bias[h * dim + d])),
+//   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   (the read-out sees the token's own write)
+// launch_stack_delta_scan leaves o in o32 [tokens, heads * vdim]; launch_stack_delta_out turns it into
+//   out[t, h, c] = o / sqrt(mean_c o^2 + eps) * norm_w[c] * sigmoid(gate_raw[t, h * vdim + c]).
+// An entry whose pos0 is 0 starts from a zero state.
+// ---------------------------------------------------------------------------------------------
+struct StackDeltaParams
+{
+    int32_t dtype = DT_BF16;
+    int32_t tokens = 0, entries = 0;
+    int32_t heads = 0, qk_heads = 0, dim = 0, vdim = 0;
+    const void* x = nullptr;          // [tokens, 2 * qk_heads * dim + heads * vdim], element type
+    const void* beta_raw = nullptr;   // element type, beta_raw[t * ld_beta + h]
+    int64_t ld_beta = 0;
+    const float* decay_raw = nullptr; // fp32 [tokens, heads * dim]
+    const float* dt_bias = nullptr;   // [heads * dim]
+    const float* a_log = nullptr;     // [heads]
+    const float* gate_raw = nullptr;  // fp32 [tokens, heads * vdim]
+    const float* norm_w = nullptr;    // [vdim]
+    float eps = 1e-5f;
+    float* state = nullptr;           // [slots, heads, dim, vdim]
+    float* o32 = nullptr;             // [tokens, heads * vdim]
+    void* out = nullptr;              // [tokens, heads * vdim], element type
+    const int32_t* ent_slot = nullptr;
+    const int32_t* ent_first = nullptr;
+    const int32_t* ent_count = nullptr;
+    const int32_t* ent_pos0 = nullptr;
+    int32_t max_count = 0;            // host: the largest ent_count of the step
+};
+int launch_stack_delta_scan(const StackDeltaParams& p, hipStream_t stream);
+int launch_stack_delta_out(const StackDeltaParams& p, hipStream_t stream);
+bool stack_delta_serves(int32_t dim, int32_t vdim);
 
 } // namespace kernels
 } // namespace tllm

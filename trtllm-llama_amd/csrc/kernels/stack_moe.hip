@@ -129,24 +129,37 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(const StackMoeParams p,
 __device__ __forceinline__ void select_token(const StackMoeParams& p, float* zr, float* cr, int lane, int t)
 {
     const int NE = p.experts + p.identity;
-    float mx = -INFINITY;
-    for (int e = lane; e < NE; e += 64)
-        mx = fmaxf(mx, zr[e]);
-    mx = wave_max(mx);
-    float sum = 0.f;
-    for (int e = lane; e < NE; e += 64)
+    if (p.score == ROUTE_SIGMOID)
     {
-        const float x = expf(zr[e] - mx);
-        zr[e] = x;
-        sum += x;
+        // every output's score by itself
+        for (int e = lane; e < NE; e += 64)
+        {
+            const float s = 1.f / (1.f + expf(-zr[e]));
+            zr[e] = s;
+            cr[e] = s + (p.correction ? p.correction[e] : 0.f);
+        }
     }
-    sum = wave_sum(sum);
-    const float inv = 1.f / sum;
-    for (int e = lane; e < NE; e += 64)
+    else
     {
-        const float s = zr[e] * inv;
-        zr[e] = s;
-        cr[e] = s + (p.correction ? p.correction[e] : 0.f);
+        float mx = -INFINITY;
+        for (int e = lane; e < NE; e += 64)
+            mx = fmaxf(mx, zr[e]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < NE; e += 64)
+        {
+            const float x = expf(zr[e] - mx);
+            zr[e] = x;
+            sum += x;
+        }
+        sum = wave_sum(sum);
+        const float inv = 1.f / sum;
+        for (int e = lane; e < NE; e += 64)
+        {
+            const float s = zr[e] * inv;
+            zr[e] = s;
+            cr[e] = s + (p.correction ? p.correction[e] : 0.f);
+        }
     }
     __builtin_amdgcn_wave_barrier();
     const int GC = p.group_count, GS = NE / GC;
@@ -293,6 +306,17 @@ __global__ __launch_bounds__(1024) void moe_route_few_kernel(const StackMoeParam
         select_token(p, sm, sm + NE, lane, t);
 }
 
+// dst[:] = w * src[:] over one row of the element type (the weight of a pair applied to the expert's input), thread `i` of `n`
+__device__ __forceinline__ void scaled_row(const StackMoeParams& p, char* dst, const char* src, float w, int i, int n)
+{
+    if (p.dtype == DT_BF16)
+        for (int c = i; c < p.width; c += n)
+            reinterpret_cast<uint16_t*>(dst)[c] = f2bf(w * bf2f(reinterpret_cast<const uint16_t*>(src)[c]));
+    else
+        for (int c = i; c < p.width; c += n)
+            reinterpret_cast<float*>(dst)[c] = w * reinterpret_cast<const float*>(src)[c];
+}
+
 // One workgroup: counts per expert, offsets, a slot per pair.  Which of an expert's slots a pair gets depends on the order of the
 // atomics; a row's product does not depend on its neighbours in a tile, so the results do not.
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const StackMoeParams p, int gather_row_bytes)
@@ -355,7 +379,9 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const StackMoeParams p, 
             continue;
         const char* src = reinterpret_cast<const char*>(p.h) + (int64_t) (i / p.top) * gather_row_bytes;
         char* dst = reinterpret_cast<char*>(p.a_sorted) + (int64_t) slot * gather_row_bytes;
-        if ((gather_row_bytes & 15) == 0)
+        if (p.weight_input)
+            scaled_row(p, dst, src, p.topk_w[i], lane, 64);
+        else if ((gather_row_bytes & 15) == 0)
             for (int b = lane * 16; b < gather_row_bytes; b += 64 * 16)
                 *reinterpret_cast<uint4*>(dst + b) = *reinterpret_cast<const uint4*>(src + b);
         else
@@ -373,7 +399,9 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const StackMoeParams p,
         return;
     const char* src = reinterpret_cast<const char*>(p.h) + (int64_t) (pair / p.top) * row_bytes;
     char* dst = reinterpret_cast<char*>(p.a_sorted) + (int64_t) slot * row_bytes;
-    if ((row_bytes & 15) == 0)
+    if (p.weight_input)
+        scaled_row(p, dst, src, p.topk_w[pair], threadIdx.x, 256);
+    else if ((row_bytes & 15) == 0)
     {
         for (int i = threadIdx.x * 16; i < row_bytes; i += 256 * 16)
             *reinterpret_cast<uint4*>(dst + i) = *reinterpret_cast<const uint4*>(src + i);
@@ -404,7 +432,8 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const StackMoeParams p
         {
             const int slot = slot_s[k];
             const float v = slot >= 0 ? ys[(int64_t) slot * p.width + c] : ld_el<DT>(p.h, (int64_t) t * p.width + c);
-            acc = fmaf(w_s[k], v, acc);
+            acc = fmaf((p.weight_input && slot >= 0) ? 1.f : w_s[k], v, acc); // an input-weighted expert's output is summed as it is
+
         }
         y[(int64_t) t * p.width + c] = acc;
     }

@@ -82,6 +82,56 @@ __global__ __launch_bounds__(256) void embed_kernel(float* x, float* keep, const
     }
 }
 
+// x[t, :] += pair_table[row, :]: the row is a hash of (previous token, token), or the table's extra last row for a first token
+template <int DT>
+__global__ __launch_bounds__(256) void pair_embed_kernel(float* x, const int32_t* ids, const int32_t* prev, const void* table, int width,
+    int buckets, int mul_prev, int mul_cur, int copies, int64_t copy_stride)
+{
+    const int t = blockIdx.x;
+    const int pv = prev[t];
+    int64_t row = buckets;
+    if (pv >= 0)
+        row = ((int64_t) pv * mul_prev + (int64_t) ids[t] * mul_cur) % buckets;
+    for (int c = threadIdx.x; c < width; c += blockDim.x)
+    {
+        const float v = El<DT>::ld(table, row * width + c);
+        for (int k = 0; k < copies; ++k)
+            x[k * copy_stride + (int64_t) t * width + c] += v;
+    }
+}
+
+// Token shift.  Workgroups [0, tokens): rows behind their entry's first read the step's own rows.  Workgroups [tokens, tokens +
+// entries): an entry's first row, which reads the sequence's carried row, and the new carry - one thread per (entry, channel) reads
+// the old carry before it writes, so the launch has no ordering between workgroups to keep.
+template <int DT>
+__global__ __launch_bounds__(256) void token_shift_kernel(const StackShiftParams p)
+{
+    const int W = p.width;
+    if ((int) blockIdx.x < p.tokens)
+    {
+        const int t = blockIdx.x, e = p.tok_entry[t];
+        if (p.tok_pos[t] == p.ent_pos0[e])
+            return;
+        for (int c = threadIdx.x; c < W; c += 256)
+        {
+            const float a = p.n[(int64_t) t * W + c], b = p.n[(int64_t) (t - 1) * W + c];
+            El<DT>::st(p.h, (int64_t) t * W + c, a + (b - a) * p.mu[c]);
+        }
+        return;
+    }
+    const int e = blockIdx.x - p.tokens;
+    const int first = p.ent_first[e], last = first + p.ent_count[e] - 1;
+    float* carry = p.carry + (int64_t) p.ent_slot[e] * W;
+    const bool fresh = p.ent_pos0[e] == 0;
+    for (int c = threadIdx.x; c < W; c += 256)
+    {
+        const float b = fresh ? 0.f : carry[c];
+        const float a = p.n[(int64_t) first * W + c];
+        El<DT>::st(p.h, (int64_t) first * W + c, a + (b - a) * p.mu[c]);
+        carry[c] = p.n[(int64_t) last * W + c];
+    }
+}
+
 // Hyper-connected residual streams: one workgroup per row; the combined row u stays in LDS between the sum of squares and the
 // scaling, the streams are read and written once.
 constexpr int HY_T = 256, HY_MAXS = 8;
@@ -141,12 +191,18 @@ __global__ __launch_bounds__(HY_T) void hyper_norm_kernel(const StackHyperParams
         u_s[c] = u;
         ss += u * u;
     }
-    if (!p.h)
+    if (!p.h && !p.h32)
         return;
     ss = block_sum(ss, red);
     const float inv = 1.f / sqrtf(ss / (float) p.width + p.eps);
     for (int c = tid; c < p.width; c += HY_T)
-        El<DT>::st(p.h, (int64_t) blockIdx.x * p.width + c, u_s[c] * inv * p.w[c]);
+    {
+        const float v = u_s[c] * inv * p.w[c];
+        if (p.h)
+            El<DT>::st(p.h, (int64_t) blockIdx.x * p.width + c, v);
+        if (p.h32)
+            p.h32[(int64_t) blockIdx.x * p.width + c] = v;
+    }
 }
 
 __global__ __launch_bounds__(256) void pass_entry_kernel(float* x, const float* add, const float* row, int64_t n, int width)
@@ -277,10 +333,11 @@ __global__ __launch_bounds__(256) void rope_kv_kernel(const StackAttnParams p)
             El<DT>::st(p.k_pool, (((int64_t) blk * (p.kv_heads * p.maps) + gm) * p.page + off) * D + d, v);
         }
     }
+    const int v_col = p.values_are_keys ? nq : nq + nk; // a layer without a value projection keeps its keys as projected
     for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < nv; i += gridDim.y * blockDim.x)
     {
         const int g = i / p.vdim, c = i % p.vdim;
-        El<DT>::st(p.v_pool, (((int64_t) blk * p.kv_heads + g) * p.vdim + c) * p.page + off, El<DT>::ld(p.proj, row + nq + nk + i));
+        El<DT>::st(p.v_pool, (((int64_t) blk * p.kv_heads + g) * p.vdim + c) * p.page + off, El<DT>::ld(p.proj, row + v_col + i));
     }
 }
 
@@ -302,7 +359,7 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const StackAttnParams p)
     const int64_t row = (int64_t) t * p.ldp;
     if (vec >= nqv + nkv)
     {
-        const int g = vec - nqv - nkv, col0 = (nqv + nkv) * D + g * p.vdim;
+        const int g = vec - nqv - nkv, col0 = (p.values_are_keys ? nqv : nqv + nkv) * D + g * p.vdim;
         for (int c = lane; c < p.vdim; c += 64)
         {
             float v = El<DT>::ld(p.proj, row + col0 + c);
@@ -332,11 +389,14 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const StackAttnParams p)
     float inv = 1.f;
     if (p.qk_unit_norm)
         inv = 1.f / sqrtf(wave_sum(ss) / (float) D + p.eps);
+    const float* nw = p.qk_unit_norm ? (vec < nqv ? p.q_norm_w : p.k_norm_w) : nullptr;
 #pragma unroll
     for (int k = 0; k < PREP_EPL; ++k)
     {
         const int d = lane + 64 * k;
         float x = v[k] * inv;
+        if (nw && d < D)
+            x *= nw[d];
         const float other = __shfl_xor(x, 1, 64); // pairs (2i, 2i + 1): lane parity = dimension parity
         if (d < p.rot_dims)
         {
@@ -456,7 +516,10 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
     const float r1 = p.log_r1 ? p.log_r1[h] : 0.f, r2 = p.log_r1 ? p.log_r2[h] : 0.f;
     const bool sigm = p.weights == WEIGHTS_SIGMOID;
     const float wb = sigm && p.wbias ? p.wbias[h] : 0.f;
-    for (int k0 = k_lo; k0 < nkeys; k0 += AT)
+    // kept first keys that lie before the window: a segment of their own ahead of the window's
+    const int keep_hi = (p.mask == MASK_WINDOW && p.mask_keep > 0) ? (p.mask_keep < k_lo ? p.mask_keep : k_lo) : 0;
+    for (int seg = keep_hi > 0 ? 0 : 1; seg < 2; ++seg)
+    for (int k0 = seg ? k_lo : 0, nkeys = seg ? pos + 1 : keep_hi; k0 < nkeys; k0 += AT)
     {
         const int kj = k0 + tid;
         float s[MAPS];
@@ -552,7 +615,7 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
             fin[m] = 1.f / l_run[m];
     }
     float og = 1.f;
-    if (p.out_gate)
+    if (p.out_gate && !p.gate_wide)
         og = 1.f / (1.f + expf(-El<DT>::ld(p.out_gate, (int64_t) t * p.ld_gate + h)));
     float o[A_CPT], ss = 0.f;
 #pragma unroll
@@ -576,7 +639,157 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
 #pragma unroll
     for (int c = 0; c < A_CPT; ++c)
         if (tid + c * AT < V)
+        {
+            if (p.out_gate && p.gate_wide)
+                og = 1.f / (1.f + expf(-El<DT>::ld(p.out_gate, (int64_t) t * p.ld_gate + (int64_t) h * V + tid + c * AT)));
             El<DT>::st(p.out, ((int64_t) t * p.heads + h) * V + tid + c * AT, o[c] * mul * og);
+        }
+}
+
+// Talking heads, general form: one workgroup per row holds ALL heads, because a head's final weight on a key mixes every head's
+// normalised weight on it.  Two passes over the visible keys, 128 at a time by one thread per key: the first leaves every head's
+// running maximum and denominator (sink included); the second recomputes the scores, normalises, mixes w'_h = sum_g talk[h, g] w_g per
+// key in the thread that owns it, and multiplies with the values of head h's own key/value head, one thread per output channel of
+// the whole row (heads * vdim / TK_T of them per thread).  One map, softmax weights; any dim, heads * vdim <= TK_T * TK_CPT.
+constexpr int TK_T = 256, TK_CPT = 16, TK_MAXH = 64;
+
+template <int DT>
+__global__ __launch_bounds__(TK_T) void attn_talk_kernel(const StackAttnParams p)
+{
+    extern __shared__ float sm[];
+    const int H = p.heads, G = p.kv_heads, D = p.dim, V = p.vdim, per = H / G;
+    float* qs = sm;                 // [H][D]
+    float* ws = qs + H * D;         // [H][TK_T] normalised weights of the block's keys
+    float* wm = ws + H * TK_T;      // [H][TK_T] the same, mixed across heads
+    float* tk = wm + H * TK_T;      // [H][H]
+    float* mh = tk + H * H;         // [H] running maxima
+    float* lh = mh + H;             // [H] denominators
+    float* red = lh + H;            // [32]
+    __shared__ int blk_of[TK_T];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int e = p.tok_entry[t], pos = p.tok_pos[t];
+    const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
+    for (int i = tid; i < H * D; i += TK_T)
+        qs[i] = El<DT>::ld(p.q, (int64_t) t * H * D + i);
+    for (int i = tid; i < H * H; i += TK_T)
+        tk[i] = p.talk ? p.talk[i] : ((i / H == i % H) ? 1.f : 0.f);
+    for (int i = tid; i < H; i += TK_T)
+    {
+        mh[i] = -INFINITY;
+        lh[i] = 0.f;
+    }
+    __syncthreads();
+    int k_lo = 0;
+    if (p.mask == MASK_WINDOW)
+        k_lo = pos - p.mask_size + 1 > 0 ? pos - p.mask_size + 1 : 0;
+    else if (p.mask == MASK_CHUNK)
+        k_lo = pos / p.mask_size * p.mask_size;
+    const int keep_hi = (p.mask == MASK_WINDOW && p.mask_keep > 0) ? (p.mask_keep < k_lo ? p.mask_keep : k_lo) : 0;
+    float acc[TK_CPT];
+#pragma unroll
+    for (int c = 0; c < TK_CPT; ++c)
+        acc[c] = 0.f;
+    for (int pass = 0; pass < 2; ++pass)
+    {
+        if (pass == 1)
+        {
+            // every head's denominator takes its sink; from here lh holds 1 / denominator relative to mh
+            __syncthreads();
+            for (int h = tid; h < H; h += TK_T)
+            {
+                float m = mh[h], l = lh[h];
+                if (p.sink)
+                {
+                    const float sk = p.sink[h], mf = fmaxf(m, sk);
+                    l = l * expf(m - mf) + expf(sk - mf);
+                    m = mf;
+                }
+                mh[h] = m;
+                lh[h] = 1.f / l;
+            }
+            __syncthreads();
+        }
+        for (int seg = keep_hi > 0 ? 0 : 1; seg < 2; ++seg)
+            for (int k0 = seg ? k_lo : 0, nkeys = seg ? pos + 1 : keep_hi; k0 < nkeys; k0 += TK_T)
+            {
+                const int kj = k0 + tid;
+                const bool live = kj < nkeys;
+                int blk = 0;
+                if (live)
+                    blk = table[kj / p.page];
+                const int off = kj % p.page;
+                blk_of[tid] = blk;
+                for (int g = 0; g < G; ++g)
+                {
+                    // a key row is read once per key/value head and serves the query heads of its group
+                    const int64_t kb = (((int64_t) blk * G + g) * p.page + off) * D;
+                    for (int hh = 0; hh < per; ++hh)
+                    {
+                        const int h = g * per + hh;
+                        float a = -INFINITY;
+                        if (live)
+                        {
+                            a = 0.f;
+                            for (int d = 0; d < D; ++d)
+                                a += qs[h * D + d] * El<DT>::ld(p.k_pool, kb + d);
+                            a *= p.scale;
+                        }
+                        if (pass == 0)
+                        {
+                            const float bm = block_max(a, red);
+                            const float mo = mh[h], mn = fmaxf(mo, bm);
+                            const float bs = block_sum(live ? expf(a - mn) : 0.f, red);
+                            __syncthreads();
+                            if (tid == 0)
+                            {
+                                lh[h] = lh[h] * expf(mo - mn) + bs;
+                                mh[h] = mn;
+                            }
+                            __syncthreads();
+                        }
+                        else
+                            ws[h * TK_T + tid] = live ? expf(a - mh[h]) * lh[h] : 0.f;
+                    }
+                }
+                if (pass == 0)
+                    continue;
+                // mix across heads for this thread's key: its own column of ws, which it wrote itself, into wm
+                for (int h = 0; h < H; ++h)
+                {
+                    float m = 0.f;
+                    for (int g = 0; g < H; ++g)
+                        m = fmaf(tk[h * H + g], ws[g * TK_T + tid], m);
+                    wm[h * TK_T + tid] = m;
+                }
+                __syncthreads();
+                const int nb = nkeys - k0 < TK_T ? nkeys - k0 : TK_T;
+#pragma unroll
+                for (int c = 0; c < TK_CPT; ++c)
+                {
+                    const int oc = tid + c * TK_T;
+                    if (oc >= H * V)
+                        break;
+                    const int h = oc / V, ch = oc % V, g = h / per;
+                    float a = acc[c];
+                    for (int j = 0; j < nb; ++j)
+                        a += wm[h * TK_T + j]
+                            * El<DT>::ld(p.v_pool, (((int64_t) blk_of[j] * G + g) * V + ch) * p.page + (k0 + j) % p.page);
+                    acc[c] = a;
+                }
+                __syncthreads();
+            }
+    }
+#pragma unroll
+    for (int c = 0; c < TK_CPT; ++c)
+    {
+        const int oc = tid + c * TK_T;
+        if (oc >= H * V)
+            break;
+        float og = 1.f;
+        if (p.out_gate)
+            og = 1.f / (1.f + expf(-El<DT>::ld(p.out_gate, (int64_t) t * p.ld_gate + (p.gate_wide ? oc : oc / V))));
+        El<DT>::st(p.out, (int64_t) t * H * V + oc, acc[c] * og);
+    }
 }
 
 // ------------------------------------------------------------------------------------------------------------------ HGRN2
@@ -846,6 +1059,45 @@ int launch_stack_embed(float* x, float* keep, const int32_t* ids, const void* ta
     return launched("stack_embed");
 }
 
+int launch_stack_pair_embed(float* x, const int32_t* ids, const int32_t* prev, const void* pair_table, int32_t dtype, int32_t tokens,
+    int32_t width, int32_t buckets, int32_t mul_prev, int32_t mul_cur, hipStream_t stream, int32_t copies, int64_t copy_stride)
+{
+    if (tokens <= 0)
+        return 0;
+    if (!known_dtype(dtype, "stack_pair_embed"))
+        return -1;
+    if (buckets < 1 || !ids || !prev || !pair_table || !x)
+    {
+        set_error("stack_pair_embed: %d buckets, or a missing operand", buckets);
+        return -1;
+    }
+    if (dtype == DT_BF16)
+        hipLaunchKernelGGL((pair_embed_kernel<DT_BF16>), dim3(tokens), dim3(256), 0, stream, x, ids, prev, pair_table, width, buckets, mul_prev,
+            mul_cur, copies, copy_stride);
+    else
+        hipLaunchKernelGGL((pair_embed_kernel<DT_FLOAT>), dim3(tokens), dim3(256), 0, stream, x, ids, prev, pair_table, width, buckets, mul_prev,
+            mul_cur, copies, copy_stride);
+    return launched("stack_pair_embed");
+}
+
+int launch_stack_token_shift(const StackShiftParams& p, hipStream_t stream)
+{
+    if (p.tokens <= 0 || p.entries <= 0)
+        return 0;
+    if (!known_dtype(p.dtype, "stack_token_shift"))
+        return -1;
+    if (p.width < 1 || !p.n || !p.mu || !p.carry || !p.h || !p.tok_entry || !p.tok_pos || !p.ent_slot || !p.ent_first || !p.ent_count || !p.ent_pos0)
+    {
+        set_error("stack_token_shift: width %d, or a missing operand", p.width);
+        return -1;
+    }
+    if (p.dtype == DT_BF16)
+        hipLaunchKernelGGL((token_shift_kernel<DT_BF16>), dim3(p.tokens + p.entries), dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL((token_shift_kernel<DT_FLOAT>), dim3(p.tokens + p.entries), dim3(256), 0, stream, p);
+    return launched("stack_token_shift");
+}
+
 namespace
 {
 // The form for rows of a multiple of 4 up to HV_K * 4096 elements: up to 1024 threads, a thread owns HV_K float4 columns of every
@@ -919,7 +1171,7 @@ __global__ __launch_bounds__(1024) void hyper_norm_vec_kernel(const StackHyperPa
             reinterpret_cast<float4*>(p.sum_out + (int64_t) t * p.width)[c4] = acc;
         ss += acc.x * acc.x + acc.y * acc.y + acc.z * acc.z + acc.w * acc.w;
     }
-    if (!p.h)
+    if (!p.h && !p.h32)
         return;
     ss = block_sum(ss, red);
     const float inv = 1.f / sqrtf(ss / (float) p.width + p.eps);
@@ -931,6 +1183,10 @@ __global__ __launch_bounds__(1024) void hyper_norm_vec_kernel(const StackHyperPa
         {
             const float4 w = reinterpret_cast<const float4*>(p.w)[c4];
             const int64_t o = (int64_t) blockIdx.x * p.width + 4 * c4;
+            if (p.h32)
+                *reinterpret_cast<float4*>(p.h32 + o) = make_float4(u[k].x * inv * w.x, u[k].y * inv * w.y, u[k].z * inv * w.z, u[k].w * inv * w.w);
+            if (!p.h)
+                continue;
             if (DT == DT_BF16)
                 *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.h) + o)
                     = make_uint2((uint32_t) f2bf(u[k].x * inv * w.x) | ((uint32_t) f2bf(u[k].y * inv * w.y) << 16),
@@ -963,13 +1219,14 @@ int launch_stack_hyper_norm(const StackHyperParams& p, hipStream_t stream)
         return 0;
     if (!known_dtype(p.dtype, "stack_hyper_norm"))
         return -1;
-    if (p.streams < 1 || p.streams > HY_MAXS || p.width < 1 || !p.x || (p.y && (!p.mix || !p.out)) || (p.h && !p.w))
+    if (p.streams < 1 || p.streams > HY_MAXS || p.width < 1 || !p.x || (p.y && (!p.mix || !p.out)) || ((p.h || p.h32) && !p.w))
     {
         set_error("stack_hyper_norm: %d streams (1 .. %d) of width %d, or a missing operand", p.streams, HY_MAXS, p.width);
         return -1;
     }
     const bool al16 = !(reinterpret_cast<uintptr_t>(p.x) & 15) && !(reinterpret_cast<uintptr_t>(p.y) & 15) && !(reinterpret_cast<uintptr_t>(p.h) & 15)
-        && !(reinterpret_cast<uintptr_t>(p.w) & 15) && !(reinterpret_cast<uintptr_t>(p.sum_out) & 15) && p.stream_stride % 4 == 0;
+        && !(reinterpret_cast<uintptr_t>(p.w) & 15) && !(reinterpret_cast<uintptr_t>(p.sum_out) & 15) && !(reinterpret_cast<uintptr_t>(p.h32) & 15)
+        && p.stream_stride % 4 == 0;
     if (p.width % 4 == 0 && p.width <= HV_K * 4096 && al16)
     {
         const int nt = std::min(1024, (p.width / 4 + 63) / 64 * 64);
@@ -1066,7 +1323,8 @@ static bool attn_shape_ok(const StackAttnParams& p, const char* what)
         set_error("%s: the rotation pairs neighbours: rot_dims %d must be even and <= dim %d", what, p.rot_dims, p.dim);
         return false;
     }
-    if (p.mask < MASK_CAUSAL || p.mask > MASK_CHUNK || (p.mask != MASK_CAUSAL && p.mask_size < 1) || p.weights < WEIGHTS_SOFTMAX
+    if (p.mask < MASK_CAUSAL || p.mask > MASK_CHUNK || (p.mask != MASK_CAUSAL && p.mask_size < 1) || p.mask_keep < 0
+        || (p.mask_keep > 0 && p.mask != MASK_WINDOW) || (p.values_are_keys && p.vdim != p.dim) || p.weights < WEIGHTS_SOFTMAX
         || p.weights > WEIGHTS_SIGMOID || (p.log_r1 && !p.log_r2))
     {
         set_error("%s: mask %d of size %d, weights %d is not a form it serves", what, p.mask, p.mask_size, p.weights);
@@ -1146,6 +1404,31 @@ int launch_stack_attention_general(const StackAttnParams& p, hipStream_t stream)
         return 0;
     if (!attn_shape_ok(p, "stack_attention"))
         return -1;
+    if (p.talk)
+    {
+        const size_t lds = sizeof(float) * ((size_t) p.heads * p.dim + 2 * (size_t) p.heads * TK_T + (size_t) p.heads * p.heads + 2 * (size_t) p.heads + 32);
+        if (p.maps != 1 || p.weights != WEIGHTS_SOFTMAX || p.softcap > 0.f || p.temp || p.slope || p.log_r1 || p.head_norm || p.heads > TK_MAXH
+            || p.heads * p.vdim > TK_T * TK_CPT || lds > 150 * 1024)
+        {
+            set_error("stack_attention: talking heads go with one softmax map without penalties, up to %d heads and %d output channels "
+                      "(heads %d, vdim %d, dim %d)",
+                TK_MAXH, TK_T * TK_CPT, p.heads, p.vdim, p.dim);
+            return -1;
+        }
+        if (p.dtype == DT_BF16)
+        {
+            if (lds > 64 * 1024)
+                (void) hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_talk_kernel<DT_BF16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds);
+            hipLaunchKernelGGL((attn_talk_kernel<DT_BF16>), dim3(p.tokens), dim3(TK_T), lds, stream, p);
+        }
+        else
+        {
+            if (lds > 64 * 1024)
+                (void) hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_talk_kernel<DT_FLOAT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds);
+            hipLaunchKernelGGL((attn_talk_kernel<DT_FLOAT>), dim3(p.tokens), dim3(TK_T), lds, stream, p);
+        }
+        return launched("stack_attention (talking heads)");
+    }
     if (p.vdim > AT * A_CPT)
     {
         set_error("stack_attention: vdim %d is beyond the %d channels the general kernel keeps", p.vdim, AT * A_CPT);
@@ -1195,6 +1478,27 @@ float stack_rope_freqs(float* freq, int32_t dims, double base, double factor, do
         freq[i] = (float) f;
     }
     return factor > 0 ? (float) (0.1 * std::log(factor) + 1.0) : 1.f;
+}
+
+void stack_rope_freqs_banded(float* freq, int32_t dims, double base, double factor, double original, double low, double high)
+{
+    const double two_pi = 6.283185307179586476925286766559;
+    for (int i = 0; i < dims / 2; ++i)
+    {
+        double f = std::pow(base, -2.0 * i / dims);
+        if (factor > 0)
+        {
+            const double wave = two_pi / f;
+            if (wave > original / low)
+                f = f / factor;
+            else if (!(wave < original / high))
+            {
+                const double s = (original / wave - low) / (high - low);
+                f = (1.0 - s) * f / factor + s * f;
+            }
+        }
+        freq[i] = (float) f;
+    }
 }
 
 bool stack_hgrn2_serves(int32_t dim, int32_t vdim)

@@ -59,13 +59,13 @@ constexpr int MAX_TAPS = 16;
 template <int DT>
 __global__ __launch_bounds__(256) void ssm_conv_kernel(const StackSsmParams p)
 {
-    const int inner = p.heads * p.vdim, CH = inner + 2 * p.groups * p.state, K = p.taps;
+    const int inner = p.heads * p.vdim, CH = p.conv_channels > 0 ? p.conv_channels : inner + 2 * p.groups * p.state, K = p.taps;
     const int c = blockIdx.y * 256 + threadIdx.x;
     if (c >= CH)
         return;
     const float* w = p.conv_w + (int64_t) c * K;
-    const float bias = p.conv_b[c];
-    const int64_t col = inner + c; // the convolution's inputs sit behind the z columns
+    const float bias = p.conv_b ? p.conv_b[c] : 0.f;
+    const int64_t col = (p.conv_channels > 0 ? p.conv_col : inner) + c; // mamba2: the convolution's inputs sit behind the z columns
     if ((int) blockIdx.x < p.tokens)
     {
         const int t = blockIdx.x, e = p.tok_entry[t];
@@ -406,9 +406,18 @@ int launch_stack_ssm_conv(const StackSsmParams& p, hipStream_t stream)
 {
     if (p.tokens <= 0 || p.entries <= 0)
         return 0;
-    if (!ssm_ok(p, "stack_ssm_conv"))
+    if (p.conv_channels > 0)
+    {
+        // the convolution alone, over a range of columns of another layer kind's projection
+        if ((p.dtype != DT_BF16 && p.dtype != DT_FLOAT) || p.taps < 1 || p.taps > MAX_TAPS || p.conv_col < 0 || !p.conv_w || !p.conv_state || !p.xbc)
+        {
+            set_error("stack_ssm_conv: %d channels, %d taps (1 .. %d), or a missing operand", p.conv_channels, p.taps, MAX_TAPS);
+            return -1;
+        }
+    }
+    else if (!ssm_ok(p, "stack_ssm_conv"))
         return -1;
-    const int CH = p.heads * p.vdim + 2 * p.groups * p.state;
+    const int CH = p.conv_channels > 0 ? p.conv_channels : p.heads * p.vdim + 2 * p.groups * p.state;
     const dim3 grid(p.tokens + p.entries, (CH + 255) / 256);
     if (p.dtype == DT_BF16)
         hipLaunchKernelGGL((ssm_conv_kernel<DT_BF16>), grid, dim3(256), 0, stream, p);

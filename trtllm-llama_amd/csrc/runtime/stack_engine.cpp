@@ -53,7 +53,8 @@ enum MixerKind
     MIX_ATTENTION = 0,
     MIX_HGRN2 = 1,
     MIX_LATENT = 2,
-    MIX_MAMBA2 = 3
+    MIX_MAMBA2 = 3,
+    MIX_DELTA = 4
 };
 enum MlpKind
 {
@@ -72,7 +73,7 @@ struct Layer
     int heads = 0, kv_heads = 0, dim = 0, vdim = 0, maps = 1, ff = 0, head_norm = 0;
     double diff = 0, scale = 1, softcap = 0;
     int rot_dims = 0;
-    double rot_base = 10000, rot_factor = 0, rot_original = 0, rot_fast = 0, rot_slow = 0;
+    double rot_base = 10000, rot_factor = 0, rot_original = 0, rot_fast = 0, rot_slow = 0, rot_low = 1, rot_high = 4;
     // derived
     int n_q = 0, n_k = 0, n_v = 0, n_mix = 0, n_ctx = 0; // columns of P1: q | k (or f) | v | rg1
     float lambda = 0.f, mscale = 1.f;
@@ -88,12 +89,17 @@ struct Layer
     int groups = 1, taps = 0, ssm_norm_groups = 1, n_conv = 0; // mamba2 (dim = state rows): B / C groups, convolution taps, parts of the output norm
     int experts = 0, identity = 0, top = 0, route_groups = 1, route_keep = 1; // moe
     double route_scale = 1;
+    int route_sigmoid = 0, route_weight_input = 0; // moe: sigmoid scores instead of a softmax; the weight scales the expert's input
+    int mask_keep = 0, talk = 0, values_are_keys = 0, gate_wide = 0, qk_norm_weight = 0, o_bias = 0, rot_banded = 0; // attention
+    int decay_rank = 0, gate_rank = 0, n_beta = 0; // delta_rule: ranks of the two low-rank projections, padded beta columns
     // device
     void *w_mix = nullptr, *w_o = nullptr, *w_gu = nullptr, *w_down = nullptr, *w_ukT = nullptr, *w_uv = nullptr;
     float *norm1 = nullptr, *norm2 = nullptr, *rg1_b = nullptr, *rg2_b = nullptr, *f_bias = nullptr, *lower = nullptr, *hnorm = nullptr,
           *freq = nullptr, *bias = nullptr, *temp = nullptr, *slope = nullptr, *r1 = nullptr, *r2 = nullptr, *sinkv = nullptr, *wbias = nullptr,
           *lat_norm = nullptr, *cq_norm = nullptr, *conv_w = nullptr, *conv_b = nullptr, *dt_bias = nullptr, *a_log = nullptr,
-          *d_skip = nullptr, *router_w = nullptr, *correction = nullptr;
+          *d_skip = nullptr, *router_w = nullptr, *correction = nullptr, *talkw = nullptr, *q_norm = nullptr, *k_norm = nullptr, *o_biasv = nullptr,
+          *shift = nullptr;
+    void *w_a2 = nullptr, *w_g2 = nullptr; // delta_rule: the second halves of the decay's and the gate's low-rank projections
     void* w_uq = nullptr;
     HyperW hc[2];
 };
@@ -104,7 +110,8 @@ struct Run
     bool enters_pass = false;
     void *k_pool = nullptr, *v_pool = nullptr; // attention
     float* state = nullptr;                    // hgrn2, mamba2
-    float* conv_state = nullptr;               // mamba2: the last taps - 1 inputs of the convolution
+    float* conv_state = nullptr;               // mamba2, delta_rule: the last taps - 1 inputs of the convolution
+    float* shift_carry = nullptr;              // token shift: the sequence's last normed row, [slots, width]
 };
 
 } // namespace
@@ -135,6 +142,12 @@ struct tllm_stack
     void *xbc = nullptr, *cq = nullptr, *qfull = nullptr, *moe_a = nullptr;
     float *moe_y = nullptr, *moe_w = nullptr;
     int32_t* moe_i = nullptr;
+    // pair embedding (a hashed row per (previous token, token)) and token shift; the previous token of every slot's sequence
+    int pair_buckets = 0, pair_mul_prev = 0, pair_mul_cur = 0, token_shift = 0;
+    void* pair_table = nullptr;
+    std::vector<int32_t> last_tok;
+    float *h32 = nullptr, *dl_a = nullptr, *dl_g = nullptr;
+    int max_hd = 0;
     int max_proj = 0, max_q = 0, max_ctx = 0, max_ff = 0, max_lat = 0, max_conv = 0, max_qrank = 0, max_qfull = 0, max_top = 0, max_experts = 0, max_outputs = 0;
     int tap_tokens = 0;
 
@@ -148,7 +161,8 @@ struct tllm_stack
     }
     void free_scratch()
     {
-        void* all[] = {x, x0, o32, logits, tap, y32, h1, h2, proj, q, ctx, act, hw, lat, ints, ids_out, xbc, cq, qfull, moe_a, moe_y, moe_w, moe_i};
+        void* all[] = {x, x0, o32, logits, tap, y32, h1, h2, proj, q, ctx, act, hw, lat, ints, ids_out, xbc, cq, qfull, moe_a, moe_y, moe_w, moe_i,
+            h32, dl_a, dl_g};
         for (void* p : all)
             if (p)
                 (void) hipFree(p);
@@ -158,6 +172,7 @@ struct tllm_stack
         xbc = cq = qfull = moe_a = nullptr;
         moe_y = moe_w = nullptr;
         moe_i = nullptr;
+        h32 = dl_a = dl_g = nullptr;
     }
 };
 
@@ -304,6 +319,9 @@ int ensure_scratch(tllm_stack* s, int tokens, int want, int n_ints)
         HIP_OK(hipMalloc(&s->xbc, T * std::max(s->max_conv, 1) * es));
         HIP_OK(hipMalloc(&s->cq, T * std::max(s->max_qrank, 1) * es));
         HIP_OK(hipMalloc(&s->qfull, T * std::max(s->max_qfull, 1) * es));
+        HIP_OK(hipMalloc((void**) &s->h32, (s->token_shift ? T * wd : 1) * 4));
+        HIP_OK(hipMalloc((void**) &s->dl_a, T * std::max(s->max_hd, 1) * 4));
+        HIP_OK(hipMalloc((void**) &s->dl_g, (s->max_hd ? T * std::max(s->max_ctx, 1) : 1) * 4));
         {
             // a mixture of experts works on one row per (token, chosen expert)
             const size_t pairs = T * (size_t) std::max(s->max_top, 1);
@@ -373,6 +391,10 @@ tllm_stack_t tllm_stack_create(const char* config_text)
     s->loop_times = geti(s, "loop_times", 1);
     s->norm_offset = (float) getd(s, "norm_offset", 0.0);
     s->streams = geti(s, "streams", 1);
+    s->pair_buckets = geti(s, "pair_buckets", 0);
+    s->pair_mul_prev = geti(s, "pair_mul_prev", 0);
+    s->pair_mul_cur = geti(s, "pair_mul_cur", 0);
+    s->token_shift = geti(s, "token_shift", 0);
     const std::string block = gets(s, "block", "parallel"), residual = gets(s, "residual", "gated");
     s->sequential = block == "sequential";
     s->hyper = residual == "hyper";
@@ -394,6 +416,9 @@ tllm_stack_t tllm_stack_create(const char* config_text)
         return fail("streams: 1 to 8, more than one only with residual=hyper");
     if (s->hyper && s->loop_stop > s->loop_start)
         return fail("looped layers are built for the gated residual only");
+    if (s->pair_buckets < 0 || (s->token_shift && !s->hyper))
+        return fail("pair_buckets >= 0; the token shift is built for block=sequential");
+    s->last_tok.assign((size_t) s->slots, -1);
     if (s->loop_times < 1 || s->loop_start < 0 || s->loop_stop < s->loop_start || s->loop_stop > L)
         return fail("the loop must satisfy 0 <= loop_start <= loop_stop <= num_layers, loop_times >= 1");
     s->layers.resize(L);
@@ -410,9 +435,11 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.kind = MIX_LATENT;
         else if (kind == "mamba2")
             l.kind = MIX_MAMBA2;
+        else if (kind == "delta_rule")
+            l.kind = MIX_DELTA;
         else
         {
-            set_error("tllm_stack_create: layer %d has mixer type '%s' (attention | latent_attention | hgrn2 | mamba2)", i, kind.c_str());
+            set_error("tllm_stack_create: layer %d has mixer type '%s' (attention | latent_attention | hgrn2 | mamba2 | delta_rule)", i, kind.c_str());
             delete s;
             return nullptr;
         }
@@ -432,8 +459,8 @@ tllm_stack_t tllm_stack_create(const char* config_text)
         l.mlp = mlp == "relu2" ? MLP_RELU2 : (mlp == "moe" ? MLP_MOE : MLP_GELU_GATE);
         if (l.mlp != MLP_GELU_GATE && !s->sequential)
             return fail("the relu2 and moe feed-forwards are built for block=sequential");
-        if ((l.kind == MIX_MAMBA2 || l.weights_of >= 0) && !s->sequential)
-            return fail("mamba2 layers and shared weights are built for block=sequential");
+        if ((l.kind == MIX_MAMBA2 || l.kind == MIX_DELTA || l.weights_of >= 0) && !s->sequential)
+            return fail("mamba2 and delta_rule layers and shared weights are built for block=sequential");
         if (l.mlp == MLP_MOE && l.ff > 0)
         {
             l.experts = geti(s, p + "experts", 0);
@@ -442,6 +469,11 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.route_groups = geti(s, p + "route_groups", 1);
             l.route_keep = geti(s, p + "route_keep", l.route_groups);
             l.route_scale = getd(s, p + "route_scale", 1.0);
+            const std::string rs = gets(s, p + "route_score", "softmax"), rw = gets(s, p + "route_weight", "output");
+            if ((rs != "softmax" && rs != "sigmoid") || (rw != "output" && rw != "input"))
+                return fail("moe: route_score softmax | sigmoid, route_weight output | input");
+            l.route_sigmoid = rs == "sigmoid";
+            l.route_weight_input = rw == "input";
             const int ne = l.experts + l.identity;
             if (l.experts < 1 || l.identity < 0 || ne > 1024 || l.top < 1 || l.top > 16 || l.top > ne || l.route_groups < 1 || ne % l.route_groups
                 || l.route_keep < 1 || l.route_keep > l.route_groups)
@@ -502,11 +534,29 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.weights = wt == "sigmoid" ? WEIGHTS_SIGMOID : WEIGHTS_SOFTMAX;
             l.sink = geti(s, p + "sink", 0);
             l.out_gate = geti(s, p + "out_gate", 0);
+            l.mask_keep = geti(s, p + "mask_keep", 0);
+            l.talk = geti(s, p + "talk", 0);
+            l.values_are_keys = geti(s, p + "values_are_keys", 0);
+            l.gate_wide = geti(s, p + "gate_wide", 0);
+            l.qk_norm_weight = geti(s, p + "qk_norm_weight", 0);
+            l.o_bias = geti(s, p + "o_bias", 0);
+            const std::string rsc = gets(s, p + "rot_scaling", "yarn");
+            if (rsc != "yarn" && rsc != "banded")
+                return fail("attention: rot_scaling yarn | banded");
+            l.rot_banded = rsc == "banded";
+            l.rot_low = getd(s, p + "rot_low", 1.0);
+            l.rot_high = getd(s, p + "rot_high", 4.0);
+            if (l.rot_banded && !(l.rot_high > l.rot_low && l.rot_low > 0))
+                return fail("attention: banded frequency scaling needs 0 < rot_low < rot_high");
             if (l.mask != MASK_CAUSAL && l.mask_size < 1)
                 return fail("attention: a window or chunk mask needs mask_size >= 1");
+            if (l.mask_keep < 0 || (l.mask_keep > 0 && l.mask != MASK_WINDOW) || (l.values_are_keys && l.vdim != l.dim)
+                || (l.gate_wide && !l.out_gate) || (l.qk_norm_weight && !l.qk_norm) || (l.o_bias && !s->hyper))
+                return fail("attention: mask_keep goes with a window, values_are_keys with vdim = dim, gate_wide with out_gate, qk_norm_weight "
+                            "with qk_norm, o_bias with block=sequential");
             if (l.sink && l.weights == WEIGHTS_SIGMOID)
                 return fail("attention: a sink belongs to softmax weights");
-            l.n_gate = l.out_gate ? l.heads : 0;
+            l.n_gate = l.out_gate ? (l.gate_wide ? l.heads * l.vdim : l.heads) : 0;
             l.kv_heads = geti(s, p + "kv_heads", l.heads);
             l.maps = geti(s, p + "maps", 1);
             l.diff = getd(s, p + "diff", 0);
@@ -522,9 +572,11 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             if (l.kv_heads < 1 || l.heads % l.kv_heads || l.maps < 1 || l.maps > 2 || (l.rot_dims > 0 && (l.dim & 1)) || (l.rot_dims & 1)
                 || l.rot_dims > l.dim)
                 return fail("attention: heads must be a multiple of kv_heads, maps 1 or 2, rot_dims even and <= dim, dim even where anything turns");
+            if (l.talk && (l.maps != 1 || l.weights != WEIGHTS_SOFTMAX || l.softcap > 0 || l.head_norm || l.head_temp || l.pos_bias))
+                return fail("attention: talking heads go with one plain softmax map");
             l.n_q = l.heads * l.maps * l.dim;
             l.n_k = l.kv_heads * l.maps * l.dim;
-            l.n_v = l.kv_heads * l.vdim;
+            l.n_v = l.values_are_keys ? 0 : l.kv_heads * l.vdim; // columns of the projection; the cache holds value rows either way
         }
         else if (l.kind == MIX_MAMBA2)
         {
@@ -540,6 +592,26 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.n_k = l.n_conv;
             l.n_v = l.heads;
             s->max_conv = std::max(s->max_conv, l.n_conv);
+        }
+        else if (l.kind == MIX_DELTA)
+        {
+            l.kv_heads = geti(s, p + "kv_heads", l.heads);
+            l.taps = geti(s, p + "conv", 4);
+            l.decay_rank = geti(s, p + "decay_rank", 0);
+            l.gate_rank = geti(s, p + "gate_rank", 0);
+            if (l.kv_heads < 1 || l.heads % l.kv_heads || l.taps < 1 || l.taps > 16 || l.decay_rank < 1 || l.gate_rank < 1
+                || !stack_delta_serves(l.dim, l.vdim))
+                return fail("delta_rule: heads a multiple of kv_heads, conv 1 .. 16, decay_rank and gate_rank positive, dim up to 2048");
+            // columns of the projection: q | k | v (the convolution's channels) | beta, padded to 8 | decay latent | gate latent
+            l.n_q = l.kv_heads * l.dim;
+            l.n_k = l.kv_heads * l.dim;
+            l.n_v = l.heads * l.vdim;
+            l.n_conv = l.n_q + l.n_k + l.n_v;
+            l.n_beta = (l.heads + 7) / 8 * 8;
+            l.n_gate = l.n_beta + l.decay_rank + l.gate_rank;
+            l.n_gate = (l.n_conv + l.n_gate + 7) / 8 * 8 - l.n_conv; // rows of the element type stay 16-byte aligned
+            s->max_conv = std::max(s->max_conv, l.n_conv);
+            s->max_hd = std::max(s->max_hd, l.heads * l.dim);
         }
         else
         {
@@ -645,6 +717,12 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
         if (upload_f32(s, one.data(), one.size(), &s->ones))
             return -1;
     }
+    if (s->pair_buckets > 0)
+    {
+        t = need(s, "bigram", {s->pair_buckets + 1, Wd});
+        if (!t || upload_rows(s, {t}, &s->pair_table))
+            return -1;
+    }
     if (s->loop_stop > s->loop_start)
     {
         t = need(s, "loop.step", {s->loop_times, Wd});
@@ -676,6 +754,8 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
             continue;
         }
         if (norm_vec(p + "norm1", Wd, &l.norm1))
+            return -1;
+        if (s->token_shift && vec("shift", Wd, &l.shift))
             return -1;
         const HostTensor* rg1 = nullptr;
         if (!s->hyper)
@@ -715,17 +795,42 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
                 || vec("mix.norm", l.n_ctx, &l.hnorm))
                 return -1;
         }
+        if (l.kind == MIX_DELTA)
+        {
+            const int64_t QK = l.n_q, HV = l.n_v, HD = (int64_t) l.heads * l.dim;
+            const HostTensor *wq = need(s, p + "mix.q", {QK, Wd}), *wk = need(s, p + "mix.k", {QK, Wd}), *wv = need(s, p + "mix.v", {HV, Wd}),
+                             *wb = need(s, p + "mix.b", {l.heads, Wd}), *a1 = need(s, p + "mix.a1", {l.decay_rank, Wd}),
+                             *a2 = need(s, p + "mix.a2", {HD, l.decay_rank}), *g1 = need(s, p + "mix.g1", {l.gate_rank, Wd}),
+                             *g2 = need(s, p + "mix.g2", {HV, l.gate_rank}), *wo = need(s, p + "mix.o", {Wd, HV}),
+                             *cq = need(s, p + "mix.q.conv", {QK, l.taps}), *ck = need(s, p + "mix.k.conv", {QK, l.taps}),
+                             *cv = need(s, p + "mix.v.conv", {HV, l.taps});
+            if (!wq || !wk || !wv || !wb || !a1 || !a2 || !g1 || !g2 || !wo || !cq || !ck || !cv)
+                return -1;
+            HostTensor pad_b, pad_end; // zero rows: beta's columns up to a multiple of 8, the projection's up to a multiple of 8
+            pad_b.dims = {l.n_beta - l.heads, Wd};
+            pad_b.v.assign((size_t) pad_b.numel(), 0.f);
+            pad_end.dims = {l.n_gate - l.n_beta - l.decay_rank - l.gate_rank, Wd};
+            pad_end.v.assign((size_t) pad_end.numel(), 0.f);
+            std::vector<float> taps(cq->v);
+            taps.insert(taps.end(), ck->v.begin(), ck->v.end());
+            taps.insert(taps.end(), cv->v.begin(), cv->v.end());
+            if (upload_rows(s, {wq, wk, wv, wb, &pad_b, a1, g1, &pad_end}, &l.w_mix) || upload_rows(s, {wo}, &l.w_o) || upload_rows(s, {a2}, &l.w_a2)
+                || upload_rows(s, {g2}, &l.w_g2) || upload_f32(s, taps.data(), taps.size(), &l.conv_w) || vec("mix.dt_bias", HD, &l.dt_bias)
+                || vec("mix.A_log", l.heads, &l.a_log) || vec("mix.norm", l.vdim, &l.hnorm))
+                return -1;
+        }
+        const bool own_mix = l.kind == MIX_MAMBA2 || l.kind == MIX_DELTA; // kinds whose projection is put together above
         const bool q_latent = l.kind == MIX_LATENT && l.q_rank > 0;
-        const HostTensor* wq = l.kind == MIX_MAMBA2 ? nullptr : need(s, p + (q_latent ? "mix.dq" : "mix.q"), {l.n_q, Wd});
-        const HostTensor* wk = l.kind == MIX_MAMBA2
+        const HostTensor* wq = own_mix ? nullptr : need(s, p + (q_latent ? "mix.dq" : "mix.q"), {l.n_q, Wd});
+        const HostTensor* wk = own_mix
             ? nullptr
             : need(s, p + (l.kind == MIX_ATTENTION ? "mix.k" : (l.kind == MIX_LATENT ? "mix.dkv" : "mix.f")), {l.n_k, Wd});
-        const HostTensor* wv = (l.kind == MIX_LATENT || l.kind == MIX_MAMBA2) ? nullptr : need(s, p + "mix.v", {l.n_v, Wd});
-        const HostTensor* wo = l.kind == MIX_MAMBA2 ? nullptr : need(s, p + "mix.o", {Wd, l.n_ctx});
+        const HostTensor* wv = (l.kind == MIX_LATENT || own_mix || l.values_are_keys) ? nullptr : need(s, p + "mix.v", {l.n_v, Wd});
+        const HostTensor* wo = own_mix ? nullptr : need(s, p + "mix.o", {Wd, l.n_ctx});
         const HostTensor* wg = l.n_gate ? need(s, p + "mix.g", {l.n_gate, Wd}) : nullptr;
-        if (l.kind != MIX_MAMBA2 && (!wq || !wk || (!wv && l.kind != MIX_LATENT) || !wo || (l.n_gate && !wg)))
+        if (!own_mix && (!wq || !wk || (!wv && l.kind != MIX_LATENT && !l.values_are_keys) || !wo || (l.n_gate && !wg)))
             return -1;
-        if (l.kind != MIX_MAMBA2)
+        if (!own_mix)
         {
             std::vector<const HostTensor*> rows = {wq, wk};
             if (wv)
@@ -740,7 +845,10 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
         if (l.kind == MIX_ATTENTION || l.kind == MIX_LATENT)
         {
             std::vector<float> fr((size_t) std::max(l.rot_dims / 2, 1));
-            l.mscale = stack_rope_freqs(fr.data(), l.rot_dims, l.rot_base, l.rot_factor, l.rot_original, l.rot_fast, l.rot_slow);
+            if (l.rot_banded)
+                stack_rope_freqs_banded(fr.data(), l.rot_dims, l.rot_base, l.rot_factor, l.rot_original, l.rot_low, l.rot_high), l.mscale = 1.f;
+            else
+                l.mscale = stack_rope_freqs(fr.data(), l.rot_dims, l.rot_base, l.rot_factor, l.rot_original, l.rot_fast, l.rot_slow);
             if (upload_f32(s, fr.data(), fr.size(), &l.freq))
                 return -1;
         }
@@ -789,12 +897,14 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
             }
             if (l.qkv_bias)
             {
-                const HostTensor *bq = need(s, p + "mix.q.b", {l.n_q}), *bk = need(s, p + "mix.k.b", {l.n_k}), *bv = need(s, p + "mix.v.b", {l.n_v});
-                if (!bq || !bk || !bv)
+                const HostTensor *bq = need(s, p + "mix.q.b", {l.n_q}), *bk = need(s, p + "mix.k.b", {l.n_k}),
+                                 *bv = l.values_are_keys ? nullptr : need(s, p + "mix.v.b", {l.n_v});
+                if (!bq || !bk || (!bv && !l.values_are_keys))
                     return -1;
                 std::vector<float> b(bq->v);
                 b.insert(b.end(), bk->v.begin(), bk->v.end());
-                b.insert(b.end(), bv->v.begin(), bv->v.end());
+                if (bv)
+                    b.insert(b.end(), bv->v.begin(), bv->v.end());
                 if (upload_f32(s, b.data(), b.size(), &l.bias))
                     return -1;
             }
@@ -810,9 +920,26 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
             }
             if (l.pos_bias == 2 && (vec("mix.r1", l.heads, &l.r1) || vec("mix.r2", l.heads, &l.r2)))
                 return -1;
-            if (l.sink && vec("mix.sink", l.heads, &l.sinkv))
+            if (l.sink == 1 && vec("mix.sink", l.heads, &l.sinkv))
                 return -1;
+            if (l.sink == 2)
+            {
+                // a constant sink of logit 0: the softmax denominator holds one more 1
+                const std::vector<float> zero((size_t) l.heads, 0.f);
+                if (upload_f32(s, zero.data(), zero.size(), &l.sinkv))
+                    return -1;
+            }
             if (l.weights == WEIGHTS_SIGMOID && vec("mix.pb", l.heads, &l.wbias))
+                return -1;
+            if (l.talk)
+            {
+                const HostTensor* tk = need(s, p + "mix.talk", {l.heads, l.heads});
+                if (!tk || upload_f32(s, tk->v.data(), tk->v.size(), &l.talkw))
+                    return -1;
+            }
+            if (l.qk_norm_weight && (vec("mix.q.norm", l.dim, &l.q_norm) || vec("mix.k.norm", l.dim, &l.k_norm)))
+                return -1;
+            if (l.o_bias && vec("mix.o.b", Wd, &l.o_biasv))
                 return -1;
         }
         else if (l.kind == MIX_HGRN2)
@@ -898,7 +1025,7 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
                 || alloc_zero(s, (size_t) s->blocks * l.kv_heads * s->page * l.vdim * s->es, &r.v_pool))
                 return -1;
         }
-        else if (l.kind == MIX_MAMBA2)
+        else if (l.kind == MIX_MAMBA2 || l.kind == MIX_DELTA)
         {
             void *st = nullptr, *cv = nullptr;
             if (alloc_zero(s, (size_t) s->slots * l.heads * l.dim * l.vdim * 4, &st)
@@ -913,6 +1040,13 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
             if (alloc_zero(s, (size_t) s->slots * l.heads * l.dim * l.vdim * 4, &st))
                 return -1;
             r.state = (float*) st;
+        }
+        if (s->token_shift)
+        {
+            void* cr = nullptr;
+            if (alloc_zero(s, (size_t) s->slots * s->width * 4, &cr))
+                return -1;
+            r.shift_carry = (float*) cr;
         }
     }
     s->host.clear();
@@ -989,12 +1123,12 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
             return -1;
         }
     // ---- metadata: one packed int32 image, one copy
-    const size_t n_ints = (size_t) 3 * T + (size_t) 4 * E + (size_t) E * MB + NW;
+    const size_t n_ints = (size_t) 4 * T + (size_t) 4 * E + (size_t) E * MB + NW;
     if (ensure_scratch(s, T, std::max(NW, 1), (int) n_ints))
         return -1;
     int32_t* h = s->pinned;
     int32_t *h_tok = h, *h_tent = h + T, *h_tpos = h + 2 * T, *h_first = h + 3 * T, *h_count = h_first + E, *h_pos0 = h_count + E,
-            *h_slot = h_pos0 + E, *h_table = h_slot + E, *h_want = h_table + (size_t) E * MB;
+            *h_slot = h_pos0 + E, *h_table = h_slot + E, *h_want = h_table + (size_t) E * MB, *h_prev = h_want + NW;
     std::memcpy(h_tok, b->tokens, (size_t) T * 4);
     int row = 0;
     for (int e = 0; e < E; ++e)
@@ -1007,7 +1141,10 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         {
             h_tent[row] = e;
             h_tpos[row] = b->ent_pos0[e] + i;
+            // the token before this one in its sequence (-1: none): the row above, or what the slot's sequence ended its last step with
+            h_prev[row] = i > 0 ? b->tokens[row - 1] : (b->ent_pos0[e] > 0 ? s->last_tok[(size_t) b->ent_slot[e]] : -1);
         }
+        s->last_tok[(size_t) b->ent_slot[e]] = b->tokens[row - 1];
         const int nb = (b->ent_pos0[e] + b->ent_count[e] + s->page - 1) / s->page;
         for (int j = 0; j < MB; ++j)
             h_table[(size_t) e * MB + j] = j < nb ? b->block_table[(size_t) e * MB + j] : 0;
@@ -1017,12 +1154,16 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
     HIP_OK(hipMemcpyAsync(s->ints, h, n_ints * 4, hipMemcpyHostToDevice, stream));
     const int32_t* d = s->ints;
     const int32_t *d_tok = d, *d_tent = d + T, *d_tpos = d + 2 * T, *d_first = d + 3 * T, *d_count = d_first + E, *d_pos0 = d_count + E,
-                  *d_slot = d_pos0 + E, *d_table = d_slot + E, *d_want = d_table + (size_t) E * MB;
+                  *d_slot = d_pos0 + E, *d_table = d_slot + E, *d_want = d_table + (size_t) E * MB, *d_prev = d_want + NW;
 
     const int Wd = s->width;
     const bool looped = s->loop_stop > s->loop_start;
     const int64_t stream_stride = (int64_t) T * Wd;
     if (launch_stack_embed(s->x, looped && s->loop_times > 1 ? s->x0 : nullptr, d_tok, s->embed, s->dtype, T, Wd, s->vocab, s->emb_scale, stream,
+            s->streams, stream_stride))
+        return -1;
+    if (s->pair_buckets > 0
+        && launch_stack_pair_embed(s->x, d_tok, d_prev, s->pair_table, s->dtype, T, Wd, s->pair_buckets, s->pair_mul_prev, s->pair_mul_cur, stream,
             s->streams, stream_stride))
         return -1;
     s->tap_tokens = T;
@@ -1041,6 +1182,79 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         g.ldc = l.n_mix;
         if (launch_stack_gemm(g, stream))
             return -1;
+        if (l.kind == MIX_DELTA)
+        {
+            // convolution + silu of q | k | v (and the sequence's new tail)
+            StackSsmParams sp;
+            sp.dtype = s->dtype;
+            sp.tokens = T;
+            sp.entries = E;
+            sp.taps = l.taps;
+            sp.proj = s->proj;
+            sp.ldp = l.n_mix;
+            sp.conv_w = l.conv_w;
+            sp.conv_channels = l.n_conv;
+            sp.conv_col = 0;
+            sp.conv_state = r.conv_state;
+            sp.xbc = s->xbc;
+            sp.tok_entry = d_tent;
+            sp.tok_pos = d_tpos;
+            sp.ent_slot = d_slot;
+            sp.ent_first = d_first;
+            sp.ent_count = d_count;
+            sp.ent_pos0 = d_pos0;
+            if (launch_stack_ssm_conv(sp, stream))
+                return -1;
+            // the two low-rank projections' second halves, in fp32: the decay's pre-activation and the output gate's
+            const int col_b = l.n_conv, col_a = col_b + l.n_beta, col_g = col_a + l.decay_rank;
+            StackGemmParams lr;
+            lr.dtype = s->dtype;
+            lr.out_f32 = 1;
+            lr.M = T;
+            lr.N = l.heads * l.dim;
+            lr.K = l.decay_rank;
+            lr.a = (const char*) s->proj + (size_t) col_a * s->es;
+            lr.lda = l.n_mix;
+            lr.w = l.w_a2;
+            lr.c = s->dl_a;
+            lr.ldc = lr.N;
+            if (launch_stack_gemm(lr, stream))
+                return -1;
+            lr.N = l.n_ctx;
+            lr.K = l.gate_rank;
+            lr.a = (const char*) s->proj + (size_t) col_g * s->es;
+            lr.w = l.w_g2;
+            lr.c = s->dl_g;
+            lr.ldc = lr.N;
+            if (launch_stack_gemm(lr, stream))
+                return -1;
+            StackDeltaParams dp;
+            dp.dtype = s->dtype;
+            dp.tokens = T;
+            dp.entries = E;
+            dp.heads = l.heads;
+            dp.qk_heads = l.kv_heads;
+            dp.dim = l.dim;
+            dp.vdim = l.vdim;
+            dp.x = s->xbc;
+            dp.beta_raw = (const char*) s->proj + (size_t) col_b * s->es;
+            dp.ld_beta = l.n_mix;
+            dp.decay_raw = s->dl_a;
+            dp.dt_bias = l.dt_bias;
+            dp.a_log = l.a_log;
+            dp.gate_raw = s->dl_g;
+            dp.norm_w = l.hnorm;
+            dp.eps = s->eps;
+            dp.state = r.state;
+            dp.o32 = s->o32;
+            dp.out = s->ctx;
+            dp.ent_slot = d_slot;
+            dp.ent_first = d_first;
+            dp.ent_count = d_count;
+            dp.ent_pos0 = d_pos0;
+            dp.max_count = max_count;
+            return (launch_stack_delta_scan(dp, stream) || launch_stack_delta_out(dp, stream)) ? -1 : 0;
+        }
         if (l.kind == MIX_MAMBA2)
         {
             StackSsmParams sp;
@@ -1211,6 +1425,12 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         a.log_r2 = l.r2;
         a.mask = l.mask;
         a.mask_size = l.mask_size;
+        a.mask_keep = l.mask_keep;
+        a.talk = l.talkw;
+        a.values_are_keys = l.values_are_keys;
+        a.gate_wide = l.gate_wide;
+        a.q_norm_w = l.q_norm;
+        a.k_norm_w = l.k_norm;
         a.weights = l.weights;
         a.sink = l.sinkv;
         a.wbias = l.wbias;
@@ -1228,7 +1448,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
     // residual=hyper: the sublayer result in y32 that has not yet been folded into the streams, and the launch that folds it,
     // combines the streams for the next reader and norms the combination
     const HyperW* pending = nullptr;
-    auto hyper = [&](const float* in, void* h, const float* w, float* sum_out) -> int {
+    auto hyper = [&](const float* in, void* h, const float* w, float* sum_out, float* h32 = nullptr) -> int {
         StackHyperParams hp;
         hp.dtype = s->dtype;
         hp.tokens = T;
@@ -1247,6 +1467,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         hp.w = w;
         hp.eps = s->eps;
         hp.sum_out = sum_out;
+        hp.h32 = h32;
         pending = nullptr;
         return launch_stack_hyper_norm(hp, stream);
     };
@@ -1257,7 +1478,30 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         const Layer& l = s->layers[r.layer];
         if (s->hyper)
         {
-            if (hyper(l.hc[0].in, s->h1, l.norm1, nullptr) || run_mixer(l, r))
+            if (s->token_shift)
+            {
+                // the norm leaves its row in fp32; the mixer reads it blended with the previous token's
+                StackShiftParams sh;
+                sh.dtype = s->dtype;
+                sh.tokens = T;
+                sh.entries = E;
+                sh.width = Wd;
+                sh.n = s->h32;
+                sh.mu = l.shift;
+                sh.carry = r.shift_carry;
+                sh.h = s->h1;
+                sh.tok_entry = d_tent;
+                sh.tok_pos = d_tpos;
+                sh.ent_slot = d_slot;
+                sh.ent_first = d_first;
+                sh.ent_count = d_count;
+                sh.ent_pos0 = d_pos0;
+                if (hyper(l.hc[0].in, nullptr, l.norm1, nullptr, s->h32) || launch_stack_token_shift(sh, stream))
+                    return -1;
+            }
+            else if (hyper(l.hc[0].in, s->h1, l.norm1, nullptr))
+                return -1;
+            if (run_mixer(l, r))
                 return -1;
             StackGemmParams o; // y = ctx Wo^T in fp32: the residual sum is 32-bit
             o.dtype = s->dtype;
@@ -1270,6 +1514,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
             o.w = l.w_o;
             o.c = s->y32;
             o.ldc = Wd;
+            o.bias = l.o_biasv;
             if (launch_stack_gemm(o, stream))
                 return -1;
             pending = &l.hc[0];
@@ -1298,6 +1543,8 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
                     mp.group_count = l.route_groups;
                     mp.group_keep = l.route_keep;
                     mp.scale = (float) l.route_scale;
+                    mp.score = l.route_sigmoid ? ROUTE_SIGMOID : ROUTE_SOFTMAX;
+                    mp.weight_input = l.route_weight_input;
                     mp.h = s->h1;
                     mp.router_w = l.router_w;
                     mp.correction = l.correction;
@@ -1552,6 +1799,9 @@ int64_t tllm_stack_step_bytes(tllm_stack_t s, int32_t n_tokens, int64_t context_
             const int64_t ctx = l.mask == MASK_CAUSAL ? context_tokens : std::min<int64_t>(context_tokens, (int64_t) n_entries * l.mask_size);
             bytes += ctx * ((int64_t) l.n_k + l.n_v) * s->es;
         }
+        else if (l.kind == MIX_DELTA)
+            bytes += ((int64_t) l.heads * l.dim * l.decay_rank + (int64_t) l.n_ctx * l.gate_rank) * s->es
+                + 2 * (int64_t) n_entries * ((int64_t) l.heads * l.dim * l.vdim + (int64_t) (l.taps - 1) * l.n_conv) * 4;
         else if (l.kind == MIX_MAMBA2)
             bytes += 2 * (int64_t) n_entries * ((int64_t) l.heads * l.dim * l.vdim + (int64_t) (l.taps - 1) * l.n_conv) * 4;
         else

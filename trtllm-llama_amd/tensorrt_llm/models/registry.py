@@ -6,6 +6,7 @@ import json
 import os
 
 from .llama.model import LLaMAForCausalLM
+from .narurax.model import NaruraxForCausalLM
 from .rofozen.model import RofozenForCausalLM
 from .tolenex.model import TolenexForCausalLM
 from .vetipel.model import VetipelForCausalLM
@@ -13,6 +14,7 @@ from .vetipel.model import VetipelForCausalLM
 MODEL_REGISTRY = {
     'LlamaForCausalLM': LLaMAForCausalLM,
     'LLaMAForCausalLM': LLaMAForCausalLM,
+    'Narurax': NaruraxForCausalLM,
     'Rofozen': RofozenForCausalLM,
     'Tolenex': TolenexForCausalLM,
     'Vetipel': VetipelForCausalLM,
