@@ -230,11 +230,19 @@ def channel_delta(h, w, p, m, eps):
 
 
 # ------------------------------------------------------------------------------------------------ feed-forward
+# a list here collects, per routed layer, the smallest relative gap between the last chosen logit and the first one left out
+margins = None
+
+
 def route(h, w, p, r):
     """-> (indices [n, top], weights [n, top]): the `top` largest sigmoid scores, lowest index among equals; weights not renormalised."""
-    s = sigmoid(h @ w[p + 'router'].T)
+    z = h @ w[p + 'router'].T
+    s = sigmoid(z)
     top = int(r['top'])
     idx = np.argsort(-s, axis=-1, kind='stable')[:, :top]
+    if margins is not None and s.shape[1] > top:
+        ranked = np.sort(z, axis=-1)[:, ::-1]   # the scores rise with the logits: the gap is measured where rounding acts
+        margins.append(((ranked[:, top - 1] - ranked[:, top]) / (np.abs(ranked[:, top - 1]) + np.abs(ranked[:, top]) + 1e-30)).min())
     return idx, np.take_along_axis(s, idx, axis=-1)
 
 
@@ -252,6 +260,31 @@ def moe(h, w, p, mlp):
 
 # ------------------------------------------------------------------------------------------------ the stack
 MIXERS = {'attention': attention, 'attention_2': attention_2, 'channel_delta': channel_delta}
+
+
+def logits(tokens, w, cfg):
+    return forward(tokens, w, cfg)
+
+
+def greedy(prompt, w, cfg, n_new):
+    """The greedy continuation, recomputed from scratch for every token."""
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        nxt = int(np.argmax(forward(toks, w, cfg)[-1]))
+        out.append(nxt)
+        toks.append(nxt)
+    return out
+
+
+def routing_margin(tokens, w, cfg):
+    """The smallest relative gap, over routed layers and tokens, between the logit of a chosen expert and the next one's."""
+    global margins
+    margins = []
+    try:
+        forward(tokens, w, cfg)
+        return min(margins) if margins else np.inf
+    finally:
+        margins = None
 
 
 def forward(tokens, w, cfg, taps=None):
