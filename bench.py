@@ -62,13 +62,16 @@ def parse():
     ap.add_argument('--parity-prompts', type=int, default=8, help='seeded prompts of the accuracy report')
     ap.add_argument('--cpu-tokens', type=int, default=0, help='CPU-baseline decode steps (0 = sized to ~20 s)')
     ap.add_argument('--cpu-threads', type=int, default=0)
-    ap.add_argument('--design', default='llama', choices=['llama', 'tolenex', 'vetipel', 'rofozen'],
+    ap.add_argument('--design', default='llama', choices=['llama', 'tolenex', 'vetipel', 'rofozen', 'narurax'],
                     help="tolenex: a side report instead of the headline workload - prefill and decode throughput of the Tolenex design "
                          "(bfloat16, ragged stack engine) at layer sizes of real models, beside LLaMA fp16 at equal size; "
                          "vetipel: the same report for the Vetipel design, beside Tolenex (the closest model: same engine, bfloat16) and "
                          "LLaMA fp16 at equal size")
     # (rofozen: the same report for the Rofozen design - mamba2 and latent-attention layers, dense and routed feed-forwards - beside
-    # Tolenex, the closest model: a recurrent / attention hybrid on the same engine in bfloat16, and Vetipel and LLaMA fp16 at equal size)
+    # Tolenex, the closest model: a recurrent / attention hybrid on the same engine in bfloat16, and Vetipel and LLaMA fp16 at equal size;
+    # narurax: the same report for the Narurax design - attention with kept first tokens, sinks and head-mixed weights, a per-channel gated
+    # delta rule, token shift, input-weighted sigmoid routing - beside Rofozen, the closest model: a recurrent / attention hybrid with
+    # routed experts on the same engine in bfloat16)
     ap.add_argument('--design-sizes', default='2048,4096', help='--design tolenex: comma list of model widths')
     ap.add_argument('--design-no-llama', action='store_true', help='--design tolenex: skip the LLaMA side (kernel traces of the new design alone)')
     ap.add_argument('--design-alone', action='store_true', help='--design vetipel: time that design only (kernel traces without its neighbours)')
@@ -631,6 +634,26 @@ def rofozen_config(width, layers, vocab=32000):
     return {'architecture': 'Rofozen', 'vocab': vocab, 'width': width, 'norm': {'eps': 1e-6}, 'layers': out}
 
 
+def narurax_config(width, layers, vocab=32000):
+    """A Narurax configuration with the layer sizes of a LLaMA-like model of this width: heads of 128, four query heads per key /
+    value head, windows of 512 tokens that keep the first 4, delta-rule layers with 128 x 128 states per head (half as many q / k
+    heads as value heads, 4 taps, low-rank pairs of width / 16), every feed-forward routing 4 of 32 experts of a quarter of
+    2.6875 x width.  Layers cycle attention_2 / channel_delta / attention / channel_delta."""
+    heads = width // 128
+    eff = -(-int(width * 2.6875 / 4) // 64) * 64
+    moe = {'kind': 'moe', 'expert': {'ff': eff}, 'router': {'experts': 32, 'top': 4}}
+    mask = {'size': 512, 'keep_first': 4}
+    a2 = {'heads': heads, 'kv_heads': max(heads // 4, 1), 'dim': 128, 'vdim': 128, 'scale': 128 ** -0.5, 'mask': mask,
+          'rot': {'dims': 128, 'base': 500000.0, 'scaling': {'factor': 8.0, 'low': 1.0, 'high': 4.0, 'original': 8192}}}
+    a1 = {'heads': heads, 'kv_heads': max(heads // 4, 1), 'dim': 128, 'vdim': 128, 'scale': 128 ** -0.5, 'mask': mask,
+          'rot': {'dims': 64, 'base': 500000.0}}
+    dl = {'heads': heads, 'kv_heads': max(heads // 2, 1), 'dim': 128, 'vdim': 128, 'conv': 4}
+    kinds = [('attention_2', a2), ('channel_delta', dl), ('attention', a1), ('channel_delta', dl)]
+    return {'architecture': 'Narurax', 'vocab': vocab, 'width': width, 'norm': {'eps': 1e-6},
+            'embedding': {'bigram': {'buckets': 65521, 'mul_prev': 1000003, 'mul_cur': 31}},
+            'layers': [{'type': kinds[i % 4][0], 'mixer': dict(kinds[i % 4][1]), 'mlp': dict(moe)} for i in range(layers)]}
+
+
 def time_stack_model(torch, model, vocab, S, K, W, tag, row):
     """Prefill (one step of S prompt tokens) and decode (single tokens at context S, 1 and 4 sequences per step) of a stack-engine
     model in bfloat16 through RaggedGenerationSession.step; wall clock around synchronised calls."""
@@ -676,11 +699,20 @@ def tolenex_report(torch, args, dev):
         L = args.design_layers
         cfg = tolenex_config(width, L)
         row = dict(width=width, layers=L, context=S)
-        if args.design == 'rofozen':
+        if args.design == 'narurax':
+            from tensorrt_llm.models import NaruraxForCausalLM
+            ncfg = narurax_config(width, L)
+            ranks = {i: (width // 16, width // 16) for i in range(L)}
+            time_stack_model(torch, NaruraxForCausalLM.from_random(ncfg, seed=1, ranks=ranks), ncfg['vocab'], S, K, W, 'narurax', row)
+            if args.design_alone:
+                rows.append({k: (round(v, 3) if isinstance(v, float) else v) for k, v in row.items()})
+                print(f'[bench] {rows[-1]}', file=sys.stderr, flush=True)
+                continue
+        if args.design in ('rofozen', 'narurax'):
             from tensorrt_llm.models import RofozenForCausalLM
             rcfg = rofozen_config(width, L)
             time_stack_model(torch, RofozenForCausalLM.from_random(rcfg, seed=1), rcfg['vocab'], S, K, W, 'rofozen', row)
-            if args.design_alone:
+            if args.design_alone or args.design == 'narurax':
                 rows.append({k: (round(v, 3) if isinstance(v, float) else v) for k, v in row.items()})
                 print(f'[bench] {rows[-1]}', file=sys.stderr, flush=True)
                 continue
@@ -769,7 +801,7 @@ def main():
         local = 0
     torch.cuda.set_device(local)
     dev = torch.device('cuda', local)
-    if args.design in ('tolenex', 'vetipel', 'rofozen'):
+    if args.design in ('tolenex', 'vetipel', 'rofozen', 'narurax'):
         if world != 1:
             raise SystemExit(f'--design {args.design} is a one-GPU report')
         return tolenex_report(torch, args, dev)

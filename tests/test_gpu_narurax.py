@@ -375,7 +375,8 @@ def test_keys_at_the_edge_of_a_window(kind, n, size, back, sees, dtype, D):
 @pytest.mark.parametrize('n,size,keep,p_far,sees', [(150, 20, 1, 0, True), (150, 20, 1, 1, False), (150, 20, 7, 6, True), (150, 20, 7, 7, False),
                                                    (200, 37, 32, 31, True), (200, 37, 32, 32, False), (200, 10, 64, 63, True),
                                                    (200, 10, 64, 64, False), (300, 64, 65, 64, True), (300, 64, 65, 65, False),
-                                                   (40, 1, 33, 32, True), (40, 1, 33, 33, False)])
+                                                   (40, 1, 33, 32, True), (40, 1, 33, 33, False), (700, 320, 40, 39, True),
+                                                   (700, 320, 40, 40, False)])
 @pytest.mark.parametrize('dtype,D', KINDS)
 @pytest.mark.parametrize('kind', ['attention', 'attention_2'])
 def test_the_first_tokens_that_a_window_keeps(kind, n, size, keep, p_far, sees, dtype, D):

@@ -63,11 +63,30 @@ struct HeadMods
 {
     float scale2, cap2, cap_arg, temp, slope2, r1, r2, wb2;
     int pen, sigm; // pen: any of temp / slope / r1 is set
+    int keep;      // the first `keep` keys of the sequence stay visible behind a window
 };
+
+// Which query, key and value head a launch's head index h stands for.  Ordinarily h is the query head and reads the key / value head
+// of its group.  cross_values: p.heads = query heads x kv_heads, and h = query head * kv_heads + value head - every query head's
+// weights applied to every value head's rows (the terms a mixing of weights across heads is made of).
+struct HeadMap
+{
+    int qh, kh, vh, q_heads;
+};
+__device__ __forceinline__ HeadMap head_map(const StackAttnParams& p, int h)
+{
+    HeadMap m;
+    m.q_heads = p.cross_values ? p.heads / p.kv_heads : p.heads;
+    m.qh = p.cross_values ? h / p.kv_heads : h;
+    m.kh = m.qh / (m.q_heads / p.kv_heads);
+    m.vh = p.cross_values ? h % p.kv_heads : m.kh;
+    return m;
+}
 
 __device__ __forceinline__ HeadMods head_mods(const StackAttnParams& p, int h)
 {
     constexpr float LOG2E = 1.4426950408889634f;
+    h = p.cross_values ? h / p.kv_heads : h; // per-head numbers belong to query heads
     HeadMods m;
     m.temp = p.temp ? p.temp[h] : 1.f;
     m.scale2 = p.scale * LOG2E * (p.softcap > 0.f ? 1.f : m.temp);
@@ -79,6 +98,7 @@ __device__ __forceinline__ HeadMods head_mods(const StackAttnParams& p, int h)
     m.pen = (p.slope || p.log_r1) ? 1 : 0;
     m.sigm = p.weights == WEIGHTS_SIGMOID;
     m.wb2 = m.sigm && p.wbias ? p.wbias[h] * LOG2E : 0.f;
+    m.keep = p.mask == MASK_WINDOW ? p.mask_keep : 0;
     return m;
 }
 
@@ -90,6 +110,26 @@ __device__ __forceinline__ int first_visible(const StackAttnParams& p, int pos)
     if (p.mask == MASK_CHUNK)
         return pos / p.mask_size * p.mask_size;
     return 0;
+}
+
+// The 32-key blocks a tile walks: from the block that holds its first row's first visible key up to the block of its last row;
+// with kept first keys, the blocks that hold them and lie before that range come first.  Step v of n visits block walk_block(w, v).
+struct BlockWalk
+{
+    int nkeep, lo, n;
+};
+__device__ __forceinline__ BlockWalk block_walk(const StackAttnParams& p, int first_row_pos, int nblk)
+{
+    BlockWalk w;
+    w.lo = first_visible(p, first_row_pos) / 32;
+    const int kept = (p.mask == MASK_WINDOW && p.mask_keep > 0) ? (p.mask_keep + 31) / 32 : 0;
+    w.nkeep = kept < w.lo ? kept : w.lo;
+    w.n = w.nkeep + (nblk - w.lo);
+    return w;
+}
+__device__ __forceinline__ int walk_block(const BlockWalk& w, int v)
+{
+    return v < w.nkeep ? v : v - w.nkeep + w.lo;
 }
 
 // Scores of one 32-key block of one map -> its P^T fragment, with the online-softmax state of the lane's query row brought up to
@@ -122,7 +162,7 @@ __device__ __forceinline__ uint4 softmax_block(f32x4 (&s)[2], float& m_run, floa
                 if (hm.r1 != 0.f)
                     v -= hm.r1 * __builtin_amdgcn_logf(fmaxf(1.f + hm.r2 * dist, 1e-30f));
             }
-            if (masked && (kidx > qpos || kidx < klo))
+            if (masked && (kidx > qpos || (kidx < klo && kidx >= hm.keep)))
                 v = -INFINITY;
             s[t][i] = v;
             bm = fmaxf(bm, v);
@@ -173,7 +213,7 @@ __device__ __forceinline__ float finish_factor(const StackAttnParams& p, int h, 
         return 1.f;
     if (!p.sink)
         return 1.f / L;
-    const float sk = p.sink[h] * 1.4426950408889634f, mf = fmaxf(M, sk);
+    const float sk = p.sink[p.cross_values ? h / p.kv_heads : h] * 1.4426950408889634f, mf = fmaxf(M, sk);
     const float wk = __builtin_amdgcn_exp2f(M - mf);
     return wk / (L * wk + __builtin_amdgcn_exp2f(sk - mf));
 }
@@ -207,7 +247,8 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     const int first = p.ent_first[e], pos0 = p.ent_pos0[e];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int col = lane & 15, g4 = lane >> 4;
-    const int g = h / (p.heads / p.kv_heads);
+    const HeadMap hd = head_map(p, h);
+    const int g = hd.kh, gv = hd.vh;
     const int page = p.page;
     const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
     const HeadMods hm = head_mods(p, h);
@@ -215,7 +256,7 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
     const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.v_pool);
 
     const int qrow = head_rows ? 0 : (r0 + col < count ? r0 + col : count - 1);
-    const int qhead = head_rows ? (hbase + col < p.heads ? hbase + col : p.heads - 1) : h;
+    const int qhead = head_rows ? (hbase + col < p.heads ? hbase + col : p.heads - 1) : hd.qh;
     const int qpos = pos0 + qrow;
     const int klo = first_visible(p, qpos);
     bf16x8 qf[MAPS][DK];
@@ -224,7 +265,7 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
 #pragma unroll
         for (int ks = 0; ks < DK; ++ks)
             qf[m][ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
-                reinterpret_cast<const uint16_t*>(p.q) + (((int64_t) (first + qrow) * p.heads + qhead) * MAPS + m) * D + ks * 32 + 8 * g4));
+                reinterpret_cast<const uint16_t*>(p.q) + (((int64_t) (first + qrow) * hd.q_heads + qhead) * MAPS + m) * D + ks * 32 + 8 * g4));
     const int last_row = head_rows ? 0 : (r0 + 15 < count ? r0 + 15 : count - 1);
     const int nblk = (pos0 + last_row) / 32 + 1;
     // the tile's key blocks: from the one that holds the first row's first visible key; klo_last: the last row's (the largest)
@@ -258,16 +299,19 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
                     kf[m][t][ks] = *reinterpret_cast<const uint4*>(krow + ks * 32);
             }
     };
-    const int kb0 = blk_lo + split * NW + w, kstep = ks * NW;
-    int blk = kb0 < nblk ? table[kb0 * 32 / page] : 0;
-    if (kb0 < nblk)
-        request_k(kb0, blk);
-    for (int kb = kb0; kb < nblk; kb += kstep)
+    const BlockWalk bw = block_walk(p, pos0 + r0, nblk);
+    const int vb0 = split * NW + w, kstep = ks * NW;
+    int kb_next = vb0 < bw.n ? walk_block(bw, vb0) : 0;
+    int blk = vb0 < bw.n ? table[kb_next * 32 / page] : 0;
+    if (vb0 < bw.n)
+        request_k(kb_next, blk);
+    for (int vb = vb0; vb < bw.n; vb += kstep)
     {
+        const int kb = kb_next;
         const int key0 = kb * 32, off = key0 % page;
         uint2 vlo[VT], vhi[VT];
         {
-            const uint16_t* vrow = vp + (((int64_t) blk * p.kv_heads + g) * V + col) * page + off + 4 * g4;
+            const uint16_t* vrow = vp + (((int64_t) blk * p.kv_heads + gv) * V + col) * page + off + 4 * g4;
 #pragma unroll
             for (int ct = 0; ct < VT; ++ct)
             {
@@ -286,10 +330,11 @@ __global__ __launch_bounds__(NW * 64) void attn_tile_kernel(const StackAttnParam
                 for (int ks = 0; ks < DK; ++ks)
                     s[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[m][t][ks]), qf[m][ks], s[m][t], 0, 0, 0);
             }
-        if (kb + kstep < nblk)
+        if (vb + kstep < bw.n)
         {
-            blk = table[(key0 + kstep * 32) / page];
-            request_k(kb + kstep, blk);
+            kb_next = walk_block(bw, vb + kstep);
+            blk = table[kb_next * 32 / page];
+            request_k(kb_next, blk);
         }
         uint4 pf[MAPS]; // P^T fragment of the block, 8 bfloat16 per map
         const bool masked = key0 + 31 > pos0 + r0 || key0 < klo_last; // wave-uniform
@@ -456,7 +501,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
     const int first = p.ent_first[e], pos0 = p.ent_pos0[e];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int col = lane & 15, g4 = lane >> 4;
-    const int g = h / (p.heads / p.kv_heads);
+    const HeadMap hd = head_map(p, h);
+    const int g = hd.kh, gv = hd.vh;
     const int page = p.page;
     const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
     const HeadMods hm = head_mods(p, h);
@@ -474,7 +520,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
 #pragma unroll
         for (int ks = 0; ks < DK; ++ks)
             qf[m][ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
-                reinterpret_cast<const uint16_t*>(p.q) + (((int64_t) (first + qrow) * p.heads + h) * MAPS + m) * D + ks * 32 + 8 * g4));
+                reinterpret_cast<const uint16_t*>(p.q) + (((int64_t) (first + qrow) * hd.q_heads + hd.qh) * MAPS + m) * D + ks * 32 + 8 * g4));
     const int wg_last = tile * 64 + 63 < count ? tile * 64 + 63 : count - 1;
     const int nblk = (pos0 + wg_last) / 32 + 1;
     const int my_last = r0 + 15 < count ? r0 + 15 : count - 1;
@@ -497,11 +543,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
 
     uint4 kr[KPT], vr[VPT];
     // the page id of a block is fetched one block before its rows are requested: one memory latency per block, not two in a row
-    int blk_next = table[wg_lo * 32 / page];
-    auto request = [&](int kb) {
-        const int key0 = kb * 32;
+    const BlockWalk bw = block_walk(p, pos0 + tile * 64, nblk);
+    // blocks below this index hold kept first keys, which every row sees whatever its own window (a wave whose rows start further
+    // down than the workgroup's first takes part in them too)
+    const int keep_blk = (p.mask == MASK_WINDOW && p.mask_keep > 0) ? (p.mask_keep + 31) / 32 : 0;
+    int blk_next = table[walk_block(bw, 0) * 32 / page];
+    auto request = [&](int vb) {
+        const int key0 = walk_block(bw, vb) * 32;
         const int blk = blk_next, off = key0 % page;
-        blk_next = table[kb + 1 < nblk ? (key0 + 32) / page : key0 / page];
+        blk_next = table[vb + 1 < bw.n ? walk_block(bw, vb + 1) * 32 / page : key0 / page];
 #pragma unroll
         for (int i = 0; i < KPT; ++i)
         {
@@ -518,12 +568,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
         {
             const int idx = tid + i * 256;
             if (V16 % 256 == 0 || idx < V16)
-                vr[i] = *reinterpret_cast<const uint4*>(vp + (((int64_t) blk * p.kv_heads + g) * V + idx / 4) * page + off + (idx % 4) * 8);
+                vr[i] = *reinterpret_cast<const uint4*>(vp + (((int64_t) blk * p.kv_heads + gv) * V + idx / 4) * page + off + (idx % 4) * 8);
         }
     };
-    request(wg_lo);
-    for (int kb = wg_lo; kb < nblk; ++kb)
+    request(0);
+    for (int vb = 0; vb < bw.n; ++vb)
     {
+        const int kb = walk_block(bw, vb);
 #pragma unroll
         for (int i = 0; i < KPT; ++i)
         {
@@ -539,9 +590,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const StackAttnParams
                 *reinterpret_cast<uint4*>(v_s + (idx / 4) * VP + (idx % 4) * 16) = vr[i];
         }
         __syncthreads();
-        if (kb + 1 < nblk)
-            request(kb + 1);
-        if (kb <= my_blk && kb >= my_lo)
+        if (vb + 1 < bw.n)
+            request(vb + 1);
+        if (kb <= my_blk && (kb >= my_lo || kb < keep_blk))
         {
             const int key0 = kb * 32;
             uint4 pf[MAPS];
@@ -636,7 +687,8 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const StackAttnP
     const int first = p.ent_first[e], pos0 = p.ent_pos0[e];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int col = lane & 15, g4 = lane >> 4;
-    const int g = h / (p.heads / p.kv_heads);
+    const HeadMap hd = head_map(p, h);
+    const int g = hd.kh, gv = hd.vh;
     const int page = p.page;
     const int32_t* table = p.block_table + (int64_t) e * p.max_blocks;
     const HeadMods hm = head_mods(p, h);
@@ -659,7 +711,7 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const StackAttnP
 #pragma unroll
         for (int ks = 0; ks < DK; ++ks)
             qf[rt][ks] = as_bf16x8(*reinterpret_cast<const uint4*>(
-                reinterpret_cast<const uint16_t*>(p.q) + ((int64_t) (first + qrow) * p.heads + h) * D + ks * 32 + 8 * g4));
+                reinterpret_cast<const uint16_t*>(p.q) + ((int64_t) (first + qrow) * hd.q_heads + hd.qh) * D + ks * 32 + 8 * g4));
         const int my_last = r0[rt] + 15 < count ? r0[rt] + 15 : count - 1;
         my_blk[rt] = rows_ok[rt] ? (pos0 + my_last) / 32 : -1;
         my_lo[rt] = rows_ok[rt] ? first_visible(p, pos0 + r0[rt]) / 32 : 0;
@@ -675,11 +727,15 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const StackAttnP
     const int wg_lo = first_visible(p, pos0 + tile * ROWS) / 32;
 
     uint4 kr[KPT], vr[VPT];
-    int blk_next = table[wg_lo * 32 / page];
-    auto request = [&](int kb) {
-        const int key0 = kb * 32;
+    const BlockWalk bw = block_walk(p, pos0 + tile * ROWS, nblk);
+    // blocks below this index hold kept first keys, which every row sees whatever its own window (a wave whose rows start further
+    // down than the workgroup's first takes part in them too)
+    const int keep_blk = (p.mask == MASK_WINDOW && p.mask_keep > 0) ? (p.mask_keep + 31) / 32 : 0;
+    int blk_next = table[walk_block(bw, 0) * 32 / page];
+    auto request = [&](int vb) {
+        const int key0 = walk_block(bw, vb) * 32;
         const int blk = blk_next, off = key0 % page;
-        blk_next = table[kb + 1 < nblk ? (key0 + 32) / page : key0 / page];
+        blk_next = table[vb + 1 < bw.n ? walk_block(bw, vb + 1) * 32 / page : key0 / page];
 #pragma unroll
         for (int i = 0; i < KPT; ++i)
         {
@@ -695,12 +751,13 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const StackAttnP
         {
             const int idx = tid + i * 256;
             if (V16 % 256 == 0 || idx < V16)
-                vr[i] = *reinterpret_cast<const uint4*>(vp + (((int64_t) blk * p.kv_heads + g) * V + idx / 4) * page + off + (idx % 4) * 8);
+                vr[i] = *reinterpret_cast<const uint4*>(vp + (((int64_t) blk * p.kv_heads + gv) * V + idx / 4) * page + off + (idx % 4) * 8);
         }
     };
-    request(wg_lo);
-    for (int kb = wg_lo; kb < nblk; ++kb)
+    request(0);
+    for (int vb = 0; vb < bw.n; ++vb)
     {
+        const int kb = walk_block(bw, vb);
 #pragma unroll
         for (int i = 0; i < KPT; ++i)
         {
@@ -716,12 +773,12 @@ __global__ __launch_bounds__(256) void attn_prefill_wide_kernel(const StackAttnP
                 *reinterpret_cast<uint4*>(v_s + (idx / 4) * VP + (idx % 4) * 16) = vr[i];
         }
         __syncthreads();
-        if (kb + 1 < nblk)
-            request(kb + 1);
+        if (vb + 1 < bw.n)
+            request(vb + 1);
         bool on[RT]; // wave-uniform
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-            on[rt] = kb <= my_blk[rt] && kb >= my_lo[rt];
+            on[rt] = kb <= my_blk[rt] && (kb >= my_lo[rt] || kb < keep_blk);
         if (on[0] || on[RT - 1])
         {
             const int key0 = kb * 32;
@@ -894,12 +951,13 @@ int launch_tile(const StackAttnParams& p, hipStream_t stream)
         if (p.split_ws && p.max_count <= 16 && p.tokens <= kSplitRows)
         {
             // a window or a chunk bounds the keys a row walks
-            const int span = p.mask == MASK_CAUSAL ? p.max_context : std::min(p.max_context, p.mask_size + 31);
+            const int span = p.mask == MASK_CAUSAL ? p.max_context
+                                                   : std::min(p.max_context, p.mask_size + 31 + (p.mask_keep > 0 ? p.mask_keep + 31 : 0));
             const int nblk = (span + 31) / 32;
             ks = std::min(kMaxSplits, (nblk + 2 * NW - 1) / (2 * NW));
         }
         // single decoded tokens whose heads share one key/value head and carry no per-head numbers: 16 heads are the tile's rows
-        const int head_rows = (p.max_count == 1 && p.kv_heads == 1 && MAPS == 1 && p.heads >= 8 && !p.temp && !p.slope && !p.log_r1 && !p.sink
+        const int head_rows = (p.max_count == 1 && p.kv_heads == 1 && !p.cross_values && MAPS == 1 && p.heads >= 8 && !p.temp && !p.slope && !p.log_r1 && !p.sink
                                   && !p.wbias && !p.head_norm)
             ? 1
             : 0;
@@ -965,7 +1023,7 @@ bool stack_attention_tiled(const StackAttnParams& p)
     const bool std_shape = (p.dim == 32 || p.dim == 64 || p.dim == 128) && (p.vdim == 32 || p.vdim == 64 || p.vdim == 128);
     const bool latent_shape = p.maps == 1 && p.kv_heads == 1 && ((p.dim == 160 && p.vdim == 128) || (p.dim == 320 && p.vdim == 256));
     // what only the general kernels do: head-mixed weights, a gate per channel, kept first keys under a window
-    if (p.talk || (p.out_gate && p.gate_wide) || p.mask_keep > 0)
+    if (p.talk || (p.out_gate && p.gate_wide))
         return false;
     return p.dtype == DT_BF16 && (std_shape || latent_shape) && p.page % 32 == 0 && p.max_count > 0 && p.entries > 0 && !(reinterpret_cast<uintptr_t>(p.q) & 15)
         && !(reinterpret_cast<uintptr_t>(p.k_pool) & 15) && !(reinterpret_cast<uintptr_t>(p.v_pool) & 7);
@@ -979,6 +1037,25 @@ int launch_stack_attention(const StackAttnParams& p, hipStream_t stream)
         const char* v = std::getenv("TLLM_STACK_ATTN_GENERAL"); // measurement knob: 1 = every shape on the general kernel
         return v && v[0] == '1';
     }();
+    if (!general_only && p.talk && p.pair_ws && p.maps == 1 && p.heads >= 1 && p.kv_heads >= 1 && p.heads % p.kv_heads == 0)
+    {
+        // head-mixed weights on the tile kernels: every query head's weights over every value head's rows (kv_heads x the pairs of a
+        // plain launch), then the mixing as a sum over those terms - the mixing is linear in the weights, so it commutes with P V
+        StackAttnParams c = p;
+        c.talk = nullptr;
+        c.out_gate = nullptr;
+        c.heads = p.heads * p.kv_heads;
+        c.cross_values = 1;
+        c.out = p.pair_ws;
+        if (stack_attention_tiled(c))
+        {
+            const int rc = launch_tile_d<1>(c, stream);
+            if (rc < 0)
+                return rc;
+            if (rc == 0)
+                return launch_stack_talk_combine(p, p.pair_ws, stream);
+        }
+    }
     if (!general_only && p.heads >= 1 && p.kv_heads >= 1 && p.heads % p.kv_heads == 0 && stack_attention_tiled(p))
     {
         int rc = p.maps == 2 ? launch_tile_d<2>(p, stream) : (p.maps == 1 ? launch_tile_d<1>(p, stream) : 1);

@@ -170,6 +170,13 @@ struct StackAttnParams
     // talking heads: talk [heads, heads] fp32 on the device, null = none.  After the softmax (sink included in the denominators) head
     // h's weight on key j becomes sum_g talk[h * heads + g] w_g(i, j); head h applies it to the values of its own key/value head.
     const float* talk = nullptr;
+    // cross_values (launch_stack_attention only): `heads` counts (query head, value head) pairs, query heads x kv_heads of them in
+    // this order; pair (g, c) applies query head g's weights (over the keys of g's own key head) to the rows of value head c; q holds
+    // heads / kv_heads query heads, out [tokens, heads * vdim].  The terms of head-mixed weights: launch_stack_talk_combine sums them.
+    int32_t cross_values = 0;
+    // room for those terms, [tokens, heads * kv_heads * vdim] of the element type: with it (and a shape of the tile kernels) a layer
+    // with `talk` runs as a cross_values launch plus launch_stack_talk_combine; without it, on the general kernel
+    void* pair_ws = nullptr;
     // values_are_keys: the layer has no value projection; a token's value row is its key as projected (unrotated, unnormed); vdim == dim
     int32_t values_are_keys = 0;
     // weights of the q / k norm (qk_unit_norm), fp32 [dim] each, null = plain unit RMS
@@ -202,7 +209,11 @@ constexpr int32_t WEIGHTS_SOFTMAX = 0, WEIGHTS_SIGMOID = 1;
 int launch_stack_rope_kv(const StackAttnParams& p, hipStream_t stream);
 // causal attention of the step's rows over their sequences' cache (which already holds the step's own keys)
 int launch_stack_attention(const StackAttnParams& p, hipStream_t stream);
-size_t stack_attn_workspace_floats(int32_t heads, int32_t maps, int32_t vdim); // floats of split_ws a layer of this shape needs
+size_t stack_attn_workspace_floats(int32_t heads, int32_t maps, int32_t vdim);
+// Talking heads from their terms: pairs [tokens, heads * kv_heads * vdim] holds, for query head g and value head c, a_gc = sum_j w_g(i, j)
+// v_c(j) (launch_stack_attention with cross_values).  out[t, h, :] = sigmoid gate * sum_g talk[h * heads + g] a_{g, kv(h)}, kv(h) = h /
+// (heads / kv_heads); gate: out_gate / ld_gate / gate_wide of `a` (null: none).  a.heads counts query heads here.
+int launch_stack_talk_combine(const StackAttnParams& a, const void* pairs, hipStream_t stream); // floats of split_ws a layer of this shape needs
 // frequencies of the rotation with YaRN-style scaling (factor <= 0: none): fills freq[dims / 2], returns the cos / sin multiplier
 float stack_rope_freqs(float* freq, int32_t dims, double base, double factor, double original, double fast, double slow);
 // frequencies with the three-band scaling by wavelength l = 2 pi / f: f stays where l < original / high, becomes f / factor where

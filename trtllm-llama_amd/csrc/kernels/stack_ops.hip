@@ -646,6 +646,29 @@ __global__ __launch_bounds__(AT) void attn_general_kernel(const StackAttnParams 
         }
 }
 
+// Talking heads from their terms (see launch_stack_talk_combine): one workgroup per row, the mixing matrix in LDS, one thread per
+// output channel of the row.
+template <int DT>
+__global__ __launch_bounds__(256) void talk_combine_kernel(const StackAttnParams p, const void* pairs)
+{
+    extern __shared__ float tk_s[]; // [H][H]
+    const int H = p.heads, G = p.kv_heads, V = p.vdim, per = H / G;
+    const int64_t t = blockIdx.x;
+    for (int i = threadIdx.x; i < H * H; i += 256)
+        tk_s[i] = p.talk[i];
+    __syncthreads();
+    for (int oc = threadIdx.x; oc < H * V; oc += 256)
+    {
+        const int h = oc / V, ch = oc % V, c = h / per;
+        float a = 0.f;
+        for (int g = 0; g < H; ++g)
+            a = fmaf(tk_s[h * H + g], El<DT>::ld(pairs, (t * H * G + g * G + c) * V + ch), a);
+        if (p.out_gate)
+            a *= 1.f / (1.f + expf(-El<DT>::ld(p.out_gate, t * p.ld_gate + (p.gate_wide ? oc : h))));
+        El<DT>::st(p.out, t * H * V + oc, a);
+    }
+}
+
 // Talking heads, general form: one workgroup per row holds ALL heads, because a head's final weight on a key mixes every head's
 // normalised weight on it.  Two passes over the visible keys, 128 at a time by one thread per key: the first leaves every head's
 // running maximum and denominator (sink included); the second recomputes the scores, normalises, mixes w'_h = sum_g talk[h, g] w_g per
@@ -1395,6 +1418,25 @@ int launch_stack_latent_prep(const StackAttnParams& p, int32_t qk_dim, const flo
     else
         hipLaunchKernelGGL((latent_prep_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, p, qk_dim, latent_norm_w, q_src, ldq, dkv_col);
     return launched("stack_latent_prep");
+}
+
+int launch_stack_talk_combine(const StackAttnParams& p, const void* pairs, hipStream_t stream)
+{
+    if (p.tokens <= 0)
+        return 0;
+    if (!known_dtype(p.dtype, "stack_talk_combine"))
+        return -1;
+    const size_t lds = sizeof(float) * (size_t) p.heads * p.heads;
+    if (!p.talk || !pairs || !p.out || p.heads < 1 || p.kv_heads < 1 || p.heads % p.kv_heads || p.vdim < 1 || lds > 64 * 1024)
+    {
+        set_error("stack_talk_combine: %d heads over %d key/value heads, vdim %d, or a missing operand", p.heads, p.kv_heads, p.vdim);
+        return -1;
+    }
+    if (p.dtype == DT_BF16)
+        hipLaunchKernelGGL((talk_combine_kernel<DT_BF16>), dim3(p.tokens), dim3(256), lds, stream, p, pairs);
+    else
+        hipLaunchKernelGGL((talk_combine_kernel<DT_FLOAT>), dim3(p.tokens), dim3(256), lds, stream, p, pairs);
+    return launched("stack_talk_combine");
 }
 
 int launch_stack_attention_general(const StackAttnParams& p, hipStream_t stream)

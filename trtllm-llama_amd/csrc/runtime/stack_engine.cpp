@@ -147,7 +147,8 @@ struct tllm_stack
     void* pair_table = nullptr;
     std::vector<int32_t> last_tok;
     float *h32 = nullptr, *dl_a = nullptr, *dl_g = nullptr;
-    int max_hd = 0;
+    void* pairs = nullptr; // talking heads: every query head's weights over every value head's rows, [tokens, heads * kv_heads * vdim]
+    int max_hd = 0, max_pairs = 0;
     int max_proj = 0, max_q = 0, max_ctx = 0, max_ff = 0, max_lat = 0, max_conv = 0, max_qrank = 0, max_qfull = 0, max_top = 0, max_experts = 0, max_outputs = 0;
     int tap_tokens = 0;
 
@@ -162,7 +163,7 @@ struct tllm_stack
     void free_scratch()
     {
         void* all[] = {x, x0, o32, logits, tap, y32, h1, h2, proj, q, ctx, act, hw, lat, ints, ids_out, xbc, cq, qfull, moe_a, moe_y, moe_w, moe_i,
-            h32, dl_a, dl_g};
+            h32, dl_a, dl_g, pairs};
         for (void* p : all)
             if (p)
                 (void) hipFree(p);
@@ -173,6 +174,7 @@ struct tllm_stack
         moe_y = moe_w = nullptr;
         moe_i = nullptr;
         h32 = dl_a = dl_g = nullptr;
+        pairs = nullptr;
     }
 };
 
@@ -320,6 +322,7 @@ int ensure_scratch(tllm_stack* s, int tokens, int want, int n_ints)
         HIP_OK(hipMalloc(&s->cq, T * std::max(s->max_qrank, 1) * es));
         HIP_OK(hipMalloc(&s->qfull, T * std::max(s->max_qfull, 1) * es));
         HIP_OK(hipMalloc((void**) &s->h32, (s->token_shift ? T * wd : 1) * 4));
+        HIP_OK(hipMalloc(&s->pairs, T * std::max(s->max_pairs, 1) * es));
         HIP_OK(hipMalloc((void**) &s->dl_a, T * std::max(s->max_hd, 1) * 4));
         HIP_OK(hipMalloc((void**) &s->dl_g, (s->max_hd ? T * std::max(s->max_ctx, 1) : 1) * 4));
         {
@@ -574,6 +577,8 @@ tllm_stack_t tllm_stack_create(const char* config_text)
                 return fail("attention: heads must be a multiple of kv_heads, maps 1 or 2, rot_dims even and <= dim, dim even where anything turns");
             if (l.talk && (l.maps != 1 || l.weights != WEIGHTS_SOFTMAX || l.softcap > 0 || l.head_norm || l.head_temp || l.pos_bias))
                 return fail("attention: talking heads go with one plain softmax map");
+            if (l.talk)
+                s->max_pairs = std::max(s->max_pairs, l.heads * l.kv_heads * l.vdim);
             l.n_q = l.heads * l.maps * l.dim;
             l.n_k = l.kv_heads * l.maps * l.dim;
             l.n_v = l.values_are_keys ? 0 : l.kv_heads * l.vdim; // columns of the projection; the cache holds value rows either way
@@ -999,7 +1004,7 @@ int32_t tllm_stack_finalize(tllm_stack_t s)
     size_t ws_floats = 0;
     for (const Layer& l : s->layers)
         if (l.kind == MIX_ATTENTION)
-            ws_floats = std::max(ws_floats, stack_attn_workspace_floats(l.heads, l.maps, l.vdim));
+            ws_floats = std::max(ws_floats, stack_attn_workspace_floats(l.talk ? l.heads * l.kv_heads : l.heads, l.maps, l.vdim));
         else if (l.kind == MIX_LATENT)
             ws_floats = std::max(ws_floats, stack_attn_workspace_floats(l.heads, 1, l.kv_rank));
     if (ws_floats)
@@ -1427,6 +1432,7 @@ int32_t tllm_stack_step(tllm_stack_t s, const tllm_stack_batch_t* b, float* logi
         a.mask_size = l.mask_size;
         a.mask_keep = l.mask_keep;
         a.talk = l.talkw;
+        a.pair_ws = l.talk ? s->pairs : nullptr;
         a.values_are_keys = l.values_are_keys;
         a.gate_wide = l.gate_wide;
         a.q_norm_w = l.q_norm;
