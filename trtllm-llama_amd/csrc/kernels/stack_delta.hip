@@ -49,30 +49,50 @@ inline int launched(const char* what)
 }
 
 // rows of a chunk: their q, k and decay vectors are prepared together, then every thread walks them in order
-constexpr int DL_RC = 8;
+constexpr int DL_RC = 16;
 
-// sum over the DS consecutive lanes (a power of two, <= 64) that hold the slices of one state column
+// sum over the DS consecutive lanes (a power of two, <= 64) that hold the slices of one state column; constant distances, so the
+// first steps are cross-lane moves inside a row of 16 lanes rather than trips through LDS
 __device__ __forceinline__ float slice_sum(float v, int DS)
 {
-    for (int o = 1; o < DS; o <<= 1)
-        v += __shfl_xor(v, o, 64);
+    if (DS > 1)
+        v += __shfl_xor(v, 1, 64);
+    if (DS > 2)
+        v += __shfl_xor(v, 2, 64);
+    if (DS > 4)
+        v += __shfl_xor(v, 4, 64);
+    if (DS > 8)
+        v += __shfl_xor(v, 8, 64);
+    if (DS > 16)
+        v += __shfl_xor(v, 16, 64);
+    if (DS > 32)
+        v += __shfl_xor(v, 32, 64);
     return v;
 }
 
 // One workgroup per (entry, head, group of `cols` value channels).  Thread (vl, s) = tid / DS, tid % DS keeps rows
 // [s NSZ, (s + 1) NSZ) of state column S[:, v] in registers.  Per chunk of DL_RC rows: the waves prepare unit q and k, the decay and
-// beta of every row into LDS (a wave per row, lanes over the key channels); then the recurrence runs row by row without leaving
-// the registers but for two slice sums (the column's S^T k and S^T q).  A head's columns are independent, so a launch with few
-// (entry, head) pairs cuts them over workgroups; the head norm is a pass of its own (delta_out_kernel).
+// beta of every row into LDS (a wave per row, lanes over the key channels) and every thread requests its column's values of the
+// whole chunk; then the recurrence runs row by row without leaving the registers: per row only the slice sum of S^T k sits on the
+// chain from one row to the next (four independent partial sums, then log2 DS cross-lane steps); the read-outs S^T q are left as
+// per-thread partials in the thread's own LDS slot and summed over the slices once per chunk, off that chain, so nothing goes to
+// memory inside the row loop.  A
+// head's columns are independent, so a launch with few (entry, head) pairs cuts them over workgroups; the head norm is a pass of
+// its own (delta_out_kernel).
 template <int DT, int NSZ>
-__global__ __launch_bounds__(1024) void delta_scan_kernel(const StackDeltaParams p, int DS, int cols)
+__global__ __launch_bounds__(256) void delta_scan_kernel(const StackDeltaParams p, int DS, int cols)
 {
     extern __shared__ float sm[];
     const int D = p.dim, V = p.vdim;
-    float* qs = sm;                  // [DL_RC][D]
-    float* ks = qs + DL_RC * D;      // [DL_RC][D]
-    float* gs = ks + DL_RC * D;      // [DL_RC][D]
-    float* bs = gs + DL_RC * D;      // [DL_RC]
+    const int DP = DS * NSZ;         // a row of the stage holds every slice whole: zeros past dim
+    float* qs = sm;                  // [DL_RC][DP]
+    float* ks = qs + DL_RC * DP;     // [DL_RC][DP]
+    float* gs = ks + DL_RC * DP;     // [DL_RC][DP]
+    float* bs = gs + DL_RC * DP;     // [DL_RC]
+    float* iqs = bs + DL_RC;         // [DL_RC] 1 / (|q| sqrt(dim)) and 1 / |k| of the chunk's rows
+    float* iks = iqs + DL_RC;
+    float* vs = iks + DL_RC;         // [DL_RC][threads] every thread's own value / read-out partial of a row: no other thread reads it
+    const int NT = blockDim.x;
     const int e = blockIdx.x, h = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6, nwaves = blockDim.x >> 6;
     const int s = tid % DS, vl = tid / DS, v = blockIdx.z * cols + vl;
@@ -81,82 +101,132 @@ __global__ __launch_bounds__(1024) void delta_scan_kernel(const StackDeltaParams
     const int hk = h / (p.heads / p.qk_heads);
     const int QK = p.qk_heads * D, CH = 2 * QK + p.heads * V, HD = p.heads * D, HV = p.heads * V;
     float* st = p.state + ((int64_t) p.ent_slot[e] * p.heads + h) * D * V;
+    const int d0 = s * NSZ;
     float S[NSZ];
 #pragma unroll
     for (int i = 0; i < NSZ; ++i)
-    {
-        const int d = s * NSZ + i;
-        S[i] = (live && d < D && p.ent_pos0[e] > 0) ? st[(int64_t) d * V + v] : 0.f;
-    }
+        S[i] = (live && d0 + i < D && p.ent_pos0[e] > 0) ? st[(int64_t) (d0 + i) * V + v] : 0.f;
+    constexpr int PF = NSZ < 16 ? NSZ : 16; // elements of the stage a thread fetches per round
     const float rate = expf(p.a_log[h]);
     const float q_mul = 1.f / sqrtf((float) D);
     for (int r0 = 0; r0 < count; r0 += DL_RC)
     {
         const int nr = count - r0 < DL_RC ? count - r0 : DL_RC;
         __syncthreads(); // the chunk before this one has been read
+        // every thread fetches its share of the chunk's (row, key channel) elements - q, k and the decay's pre-activation - with all
+        // of its loads in flight at once, then the decays are formed and everything lands in the stage
+        for (int base = 0; base < nr * DP; base += NT * PF)
+        {
+            float rq[PF], rk[PF], ra[PF];
+#pragma unroll
+            for (int j = 0; j < PF; ++j)
+            {
+                const int el = base + j * NT + tid, r = el / DP, d = el - r * DP;
+                const bool in = el < nr * DP && d < D;
+                const int64_t t = first + r0 + r;
+                rq[j] = in ? ld_el<DT>(p.x, t * CH + hk * D + d) : 0.f;
+                rk[j] = in ? ld_el<DT>(p.x, t * CH + QK + hk * D + d) : 0.f;
+                ra[j] = in ? p.decay_raw[t * HD + h * D + d] + p.dt_bias[h * D + d] : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < PF; ++j)
+            {
+                const int el = base + j * NT + tid, r = el / DP, d = el - r * DP;
+                if (el < nr * DP)
+                {
+                    qs[el] = rq[j];
+                    ks[el] = rk[j];
+                    gs[el] = d < D ? expf(-rate * softplus_f(ra[j])) : 0.f;
+                }
+            }
+        }
+        {
+            float rv[DL_RC];
+#pragma unroll
+            for (int r = 0; r < DL_RC; ++r)
+                rv[r] = (live && r < nr) ? ld_el<DT>(p.x, (int64_t) (first + r0 + r) * CH + 2 * QK + h * V + v) : 0.f;
+#pragma unroll
+            for (int r = 0; r < DL_RC; ++r)
+                vs[r * NT + tid] = rv[r];
+        }
+        if (tid < nr)
+            bs[tid] = 1.f / (1.f + expf(-ld_el<DT>(p.beta_raw, (int64_t) (first + r0 + tid) * p.ld_beta + h)));
+        __syncthreads();
+        // q and k stay as projected in the stage; their unit-norm factors are applied to the sums they enter
         for (int r = wid; r < nr; r += nwaves)
         {
-            const int64_t t = first + r0 + r;
             float sq = 0.f, sk = 0.f;
             for (int d = lane; d < D; d += 64)
             {
-                const float qv = ld_el<DT>(p.x, t * CH + hk * D + d), kv = ld_el<DT>(p.x, t * CH + QK + hk * D + d);
-                sq += qv * qv;
-                sk += kv * kv;
+                sq = fmaf(qs[r * DP + d], qs[r * DP + d], sq);
+                sk = fmaf(ks[r * DP + d], ks[r * DP + d], sk);
             }
-            const float iq = q_mul / sqrtf(wave_sum(sq) + 1e-6f), ik = 1.f / sqrtf(wave_sum(sk) + 1e-6f);
-            for (int d = lane; d < D; d += 64)
-            {
-                qs[r * D + d] = ld_el<DT>(p.x, t * CH + hk * D + d) * iq;
-                ks[r * D + d] = ld_el<DT>(p.x, t * CH + QK + hk * D + d) * ik;
-                gs[r * D + d] = expf(-rate * softplus_f(p.decay_raw[t * HD + h * D + d] + p.dt_bias[h * D + d]));
-            }
+            sq = wave_sum(sq);
+            sk = wave_sum(sk);
             if (lane == 0)
-                bs[r] = 1.f / (1.f + expf(-ld_el<DT>(p.beta_raw, t * p.ld_beta + h)));
+            {
+                iqs[r] = q_mul / sqrtf(sq + 1e-6f);
+                iks[r] = 1.f / sqrtf(sk + 1e-6f);
+            }
         }
         __syncthreads();
         for (int r = 0; r < nr; ++r)
         {
-            const int64_t t = first + r0 + r;
-            const float vv = live ? ld_el<DT>(p.x, t * CH + 2 * QK + h * V + v) : 0.f;
-            float dot = 0.f;
-#pragma unroll
-            for (int i = 0; i < NSZ; ++i)
             {
-                const int d = s * NSZ + i;
-                if (d < D)
+                // rows of the stage past dim hold zeros and the state rows there stay zero: no guard inside the slices
+                const float* gr = gs + r * DP + d0;
+                const float* kr = ks + r * DP + d0;
+                const float* qr = qs + r * DP + d0;
+                float part[4] = {0.f, 0.f, 0.f, 0.f};
                 {
-                    S[i] *= gs[r * D + d];
-                    dot = fmaf(S[i], ks[r * D + d], dot);
-                }
-            }
-            dot = slice_sum(dot, DS);
-            const float u = bs[r] * (vv - dot);
-            float o = 0.f;
 #pragma unroll
-            for (int i = 0; i < NSZ; ++i)
-            {
-                const int d = s * NSZ + i;
-                if (d < D)
-                {
-                    S[i] = fmaf(ks[r * D + d], u, S[i]);
-                    o = fmaf(S[i], qs[r * D + d], o);
+                    for (int i = 0; i < NSZ; i += 4)
+                    {
+                        const float4 g4 = *reinterpret_cast<const float4*>(gr + i), k4 = *reinterpret_cast<const float4*>(kr + i);
+                        S[i] *= g4.x;
+                        S[i + 1] *= g4.y;
+                        S[i + 2] *= g4.z;
+                        S[i + 3] *= g4.w;
+                        part[0] = fmaf(S[i], k4.x, part[0]);
+                        part[1] = fmaf(S[i + 1], k4.y, part[1]);
+                        part[2] = fmaf(S[i + 2], k4.z, part[2]);
+                        part[3] = fmaf(S[i + 3], k4.w, part[3]);
+                    }
                 }
+                const float dot = slice_sum((part[0] + part[1]) + (part[2] + part[3]), DS) * iks[r];
+                const float u = bs[r] * (vs[r * NT + tid] - dot) * iks[r]; // times the key's norm factor: S += k_hat u = k (u / |k|)
+                float op[4] = {0.f, 0.f, 0.f, 0.f};
+                {
+#pragma unroll
+                    for (int i = 0; i < NSZ; i += 4)
+                    {
+                        const float4 k4 = *reinterpret_cast<const float4*>(kr + i), q4 = *reinterpret_cast<const float4*>(qr + i);
+                        S[i] = fmaf(k4.x, u, S[i]);
+                        S[i + 1] = fmaf(k4.y, u, S[i + 1]);
+                        S[i + 2] = fmaf(k4.z, u, S[i + 2]);
+                        S[i + 3] = fmaf(k4.w, u, S[i + 3]);
+                        op[0] = fmaf(S[i], q4.x, op[0]);
+                        op[1] = fmaf(S[i + 1], q4.y, op[1]);
+                        op[2] = fmaf(S[i + 2], q4.z, op[2]);
+                        op[3] = fmaf(S[i + 3], q4.w, op[3]);
+                    }
+                }
+                vs[r * NT + tid] = ((op[0] + op[1]) + (op[2] + op[3])) * iqs[r];
             }
-            o = slice_sum(o, DS);
+        }
+        for (int r = 0; r < nr; ++r)
+        {
+            const float o = slice_sum(vs[r * NT + tid], DS);
             if (live && s == 0)
-                p.o32[t * HV + h * V + v] = o;
+                p.o32[(int64_t) (first + r0 + r) * HV + h * V + v] = o;
         }
     }
     if (live)
     {
 #pragma unroll
         for (int i = 0; i < NSZ; ++i)
-        {
-            const int d = s * NSZ + i;
-            if (d < D)
-                st[(int64_t) d * V + v] = S[i];
-        }
+            if (d0 + i < D)
+                st[(int64_t) (d0 + i) * V + v] = S[i];
     }
 }
 
@@ -189,7 +259,9 @@ DeltaShape delta_shape(int dim, int vdim)
 {
     (void) vdim;
     DeltaShape r;
-    for (int limit : {16, 64}) // up to 16 slices where 32 rows per thread allow it (four shuffle steps per sum), else up to a wave
+    // up to 16 slices with the fewest rows per thread that allow it (measured at dim 128: 8 rows x 16 slices beat 32 x 4 - the time
+    // of a row is the thread's own instructions, not the four cross-lane steps), else 32 rows per thread and up to a wave of slices
+    for (int limit : {16, 64})
         for (int nsz : {8, 16, 32})
         {
             int ds = 1;
@@ -205,19 +277,23 @@ template <int DT>
 int launch_scan(const StackDeltaParams& p, hipStream_t stream)
 {
     const DeltaShape sh = delta_shape(p.dim, p.vdim);
-    // columns per workgroup: the whole head, or fewer while the launch would leave most of the chip idle
-    int cols = std::min(p.vdim, 1024 / sh.ds);
+    // columns per workgroup: four waves' worth (a wave per SIMD, and the chunk's rows are prepared once for all of them), fewer
+    // while the launch would leave most of the chip idle
+    int cols = std::min(p.vdim, std::max(256 / sh.ds, 1));
     const int cus = launch_util::device_cus();
-    while (cols > 16 && (int64_t) p.entries * p.heads * ((p.vdim + cols - 1) / cols) < cus && (cols / 2) * sh.ds >= 64)
+    while (cols * sh.ds > 128 && (int64_t) p.entries * p.heads * ((p.vdim + cols - 1) / cols) * 2 <= cus)
         cols = (cols + 1) / 2;
-    const int threads = std::min(1024, (cols * sh.ds + 63) / 64 * 64);
+    const int threads = (cols * sh.ds + 63) / 64 * 64; // at most 256: cols * slices <= 256, or one column of up to 64 slices
     const dim3 grid(p.entries, p.heads, (p.vdim + cols - 1) / cols);
-    const size_t lds = sizeof(float) * ((size_t) 3 * DL_RC * p.dim + DL_RC);
+    const size_t lds = sizeof(float) * ((size_t) 3 * DL_RC * sh.ds * sh.nsz + 3 * DL_RC + (size_t) DL_RC * threads);
     switch (sh.nsz)
     {
     case 8: hipLaunchKernelGGL((delta_scan_kernel<DT, 8>), grid, dim3(threads), lds, stream, p, sh.ds, cols); break;
     case 16: hipLaunchKernelGGL((delta_scan_kernel<DT, 16>), grid, dim3(threads), lds, stream, p, sh.ds, cols); break;
-    default: hipLaunchKernelGGL((delta_scan_kernel<DT, 32>), grid, dim3(threads), lds, stream, p, sh.ds, cols); break;
+    default:
+        launch_util::ensure_dynamic_lds(reinterpret_cast<const void*>(&delta_scan_kernel<DT, 32>), 120 * 1024); // raised once, for the largest dim
+        hipLaunchKernelGGL((delta_scan_kernel<DT, 32>), grid, dim3(threads), lds, stream, p, sh.ds, cols);
+        break;
     }
     return launched("stack_delta_scan");
 }
@@ -231,7 +307,7 @@ bool delta_ok(const StackDeltaParams& p, const char* what)
     }
     if (p.heads < 1 || p.qk_heads < 1 || p.heads % p.qk_heads || !stack_delta_serves(p.dim, p.vdim))
     {
-        set_error("%s: heads %d over %d q/k heads, dim %d, vdim %d is not a shape it serves (heads a multiple of the q/k heads, dim <= 2048)",
+        set_error("%s: heads %d over %d q/k heads, dim %d, vdim %d is not a shape it serves (heads a multiple of the q/k heads, dim <= 512)",
             what, p.heads, p.qk_heads, p.dim, p.vdim);
         return false;
     }
@@ -242,7 +318,7 @@ bool delta_ok(const StackDeltaParams& p, const char* what)
 
 bool stack_delta_serves(int32_t dim, int32_t vdim)
 {
-    return dim >= 1 && vdim >= 1 && dim <= 2048 && delta_shape(dim, vdim).nsz > 0;
+    return dim >= 1 && vdim >= 1 && dim <= 512 && delta_shape(dim, vdim).nsz > 0; // 16 staged rows of q, k and the decay within 128 KiB of LDS
 }
 
 int launch_stack_delta_scan(const StackDeltaParams& p, hipStream_t stream)

@@ -606,7 +606,7 @@ tllm_stack_t tllm_stack_create(const char* config_text)
             l.gate_rank = geti(s, p + "gate_rank", 0);
             if (l.kv_heads < 1 || l.heads % l.kv_heads || l.taps < 1 || l.taps > 16 || l.decay_rank < 1 || l.gate_rank < 1
                 || !stack_delta_serves(l.dim, l.vdim))
-                return fail("delta_rule: heads a multiple of kv_heads, conv 1 .. 16, decay_rank and gate_rank positive, dim up to 2048");
+                return fail("delta_rule: heads a multiple of kv_heads, conv 1 .. 16, decay_rank and gate_rank positive, dim up to 512");
             // columns of the projection: q | k | v (the convolution's channels) | beta, padded to 8 | decay latent | gate latent
             l.n_q = l.kv_heads * l.dim;
             l.n_k = l.kv_heads * l.dim;
