@@ -13,12 +13,17 @@
  * interleaved rotary positions on the first rot_dims dimensions with YaRN-style frequency scaling, tanh soft cap, per-head RMS
  * norm of the output; optionally projection biases, unit-RMS queries and keys, a per-head temperature, a linear or logarithmic
  * distance penalty, a sliding-window or chunked mask, sigmoid weights instead of a softmax, a softmax sink, a per-head output
- * gate), "latent_attention" (keys and values expanded from one low-rank latent per token plus one rotated key part shared by the
+ * gate; a window that also keeps the sequence's first keys, values that are the keys as projected, weights mixed across heads by a
+ * learned matrix after the softmax, a gate per output channel, weighted q / k norms, three-band frequency scaling, an output bias),
+ * "latent_attention" (keys and values expanded from one low-rank latent per token plus one rotated key part shared by the
  * heads; the cache holds the latent and that part, attention runs in the absorbed form; optionally queries expanded from a normed
  * latent of their own, half-split rotation pairs with YaRN-style frequency scaling, a window or chunk mask, a softmax sink), "hgrn2"
  * (gated linear recurrence with a lower-bounded forget gate, fp32 state) and "mamba2" (selective state-space layer: a short causal
  * convolution whose last inputs are part of the state, S <- exp(-exp(A_log) dt) S + dt B x^T per head over grouped B / C, skip, gate,
- * RMS norm in parts of the row).  Feed-forwards: gated dense, relu^2, or a routed mixture of gated experts (softmax router with a
+ * RMS norm in parts of the row) and "delta_rule" (gated delta rule with a decay per key channel: q | k | v through a short causal
+ * convolution and silu, unit q and k, S <- diag(g) S, u = beta (v - S^T k), S <- S + k u^T, o = S^T q; RMS norm per head and a low-rank
+ * sigmoid gate).  The embedding may add a hashed row per (previous token, token) pair, and every mixer's normed input may be blended
+ * with the previous token's (token shift); both carry one item per sequence in its state slot.  Feed-forwards: gated dense, relu^2, or a routed mixture of gated experts (softmax router with a
  * choice correction, groups of experts of which only the best can be chosen, identity experts).  A layer may run on an earlier
  * layer's weights (layer.<i>.weights_of), with a cache / state of its own.  Two block forms: parallel sublayers on one residual whose updates are gated by
  * sigmoid(W h + b), RMS norms in groups, a range of layers optionally run several times in a row (every pass with a cache / state
@@ -47,23 +52,33 @@ typedef struct tllm_stack* tllm_stack_t;
  *   loop_start, loop_stop, loop_times (0, 0, 1: no loop), page_size (64), num_blocks, num_slots, debug_taps (0),
  *   block (parallel | sequential), residual (gated | hyper; parallel goes with gated, sequential with hyper), streams (1 .. 8),
  *   norm_offset (0: a norm weight is applied as norm_offset + stored value),
- *   per layer i: layer.<i>.type (attention | latent_attention | hgrn2 | mamba2), .heads, .dim, .vdim, .ff (0: no feed-forward),
+ *   pair_buckets (0: none; the tensor `bigram` [pair_buckets + 1, width] adds row (prev * pair_mul_prev + token * pair_mul_cur) mod
+ *     pair_buckets to a token's embedding, its last row to a sequence's first token), pair_mul_prev, pair_mul_cur,
+ *   token_shift (0 | 1: the mixer reads h + (h_prev - h) * l<i>.shift, h the normed row; sequential blocks only),
+ *   per layer i: layer.<i>.type (attention | latent_attention | hgrn2 | mamba2 | delta_rule), .heads, .dim, .vdim, .ff (0: no feed-forward),
  *     .weights_of (an earlier layer with weights of its own; sequential blocks only),
  *     .mlp (gelu_gate: W_down (gelu_tanh(W_gate h) * W_up h) | relu2: W_down relu(W_up h)^2 | moe: .experts experts
  *       W_down (silu(W_gate h) * W_up h) of size .ff plus .identity identity outputs, .top chosen per token among the .route_keep best
- *       of .route_groups equal groups, weights = softmax score * .route_scale; relu2 and moe in sequential blocks only),
+ *       of .route_groups equal groups, weights = softmax score * .route_scale; .route_score softmax | sigmoid (every output's
+ *       score by itself), .route_weight output | input (the weight multiplies the expert's input row and the outputs are summed as they
+ *       are); relu2 and moe in sequential blocks only),
  *     attention: .kv_heads, .maps (1 | 2), .diff (the constant of the second map's weight and of the output scale 1 - diff),
  *       .scale, .softcap (0: none), .head_norm (0 | 1), .rot_dims, .rot_base, .rot_factor (0: no frequency scaling),
  *       .rot_original, .rot_fast, .rot_slow, .qkv_bias (0 | 1), .qk_norm (0 | 1: q and k / their RMS over dim), .head_temp (0 | 1),
  *       .pos_bias (none | linear: slope_h = 2^(-slope_base (h + 1) / heads) | log: r1_h ln(1 + r2_h (i - j))), .slope_base (8),
- *       .mask (causal | window | chunk), .mask_size, .weights (softmax | sigmoid), .sink (0 | 1), .out_gate (0 | 1);
+ *       .mask (causal | window | chunk), .mask_size, .mask_keep (windows: the first keys every row keeps seeing), .weights (softmax |
+ *       sigmoid), .sink (0 | 1: learned per head | 2: a constant logit of 0), .out_gate (0 | 1), .gate_wide (0 | 1: a gate per output
+ *       channel), .talk (0 | 1: weights mixed across heads by mix.talk [heads, heads]), .values_are_keys (0 | 1: no value projection),
+ *       .qk_norm_weight (0 | 1: mix.q.norm / mix.k.norm [dim]), .o_bias (0 | 1), .rot_scaling (yarn | banded: .rot_low, .rot_high);
  *     latent_attention: .kv_rank, .rot_dim (size of the shared rotated part), .rot_dims (how many of them turn), .rot_base, .scale,
  *       .q_rank (0: queries straight from the input), .rot_pairing (neighbours | halves), .rot_factor / .rot_original / .rot_fast /
  *       .rot_slow, .mask, .mask_size, .sink;
- *     mamba2: .state (rows of a head's state; takes the place of .dim), .groups, .conv (taps), .ssm_norm_groups.
+ *     mamba2: .state (rows of a head's state; takes the place of .dim), .groups, .conv (taps), .ssm_norm_groups;
+ *     delta_rule: .kv_heads (q / k heads), .conv (taps), .decay_rank, .gate_rank (of the two low-rank pairs).
  * Weights are named l<i>.norm1, l<i>.norm2, l<i>.mix.{q,k,v,o,lq1,lk1,lq2,lk2} (attention; with the options also q.b, k.b, v.b,
- * temp, r1, r2, sink, pb, g), l<i>.mix.{q,dkv,dkv.norm,uk,uv,o} (latent_attention; with a query latent dq, dq.norm, uq instead of q;
+ * temp, r1, r2, sink, pb, g, talk, q.norm, k.norm, o.b), l<i>.mix.{q,dkv,dkv.norm,uk,uv,o} (latent_attention; with a query latent dq, dq.norm, uq instead of q;
  * sink), l<i>.mix.{q,f,f.b,lower,v,norm,o} (hgrn2), l<i>.mix.{in,conv,conv.b,dt_bias,A_log,D,norm,o} (mamba2),
+ * l<i>.mix.{q,k,v,q.conv,k.conv,v.conv,b,a1,a2,dt_bias,A_log,g1,g2,norm,o} (delta_rule), l<i>.shift (token shift), bigram,
  * l<i>.mlp.{gate,up,down} (moe: l<i>.mlp.e<k>.{gate,up,down}, l<i>.mlp.router, l<i>.mlp.correction), l<i>.rg1, l<i>.rg1.b, l<i>.rg2, l<i>.rg2.b (gated residual), l<i>.hc{1,2}.{in,out,mix} (hyper
  * residual; absent with one stream: the plain sum), embed, loop.step, final.norm, head; linear weights [out, in]. */
 tllm_stack_t tllm_stack_create(const char* config_text);

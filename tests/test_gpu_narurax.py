@@ -116,6 +116,9 @@ MECHANISMS = {
     'attention_window_wider_than_the_prompt': make_config([attn_layer(size=500, keep=2)]),
     'attention_many_heads': make_config([attn_layer(heads=16, kv_heads=4, dim=4, rot_dims=4)]),
     'attention_tile_64': make_config([TILED[2]], width=128),
+    'attention_tile_32_one_kv_head': make_config([attn_layer(heads=4, kv_heads=1, dim=32, rot_dims=32, size=40, keep=2)], width=128),
+    'attention_tile_128_kv_per_head': make_config([attn_layer(heads=2, kv_heads=2, dim=128, rot_dims=64, size=90, keep=35)], width=128),
+    'attention_tile_64_eight_pairs_per_head': make_config([attn_layer(heads=8, kv_heads=8, dim=64, rot_dims=16, size=0)], width=128),
     'attention2_alone_no_ff': make_config([attn2_layer()]),
     'attention2_no_scaling': make_config([attn2_layer(scaling=False)]),
     'attention2_partly_rotated': make_config([attn2_layer(dim=14, rot_dims=6)]),
@@ -146,7 +149,7 @@ MECHANISMS = {
     'width_that_is_no_multiple_of_four': make_config([attn_layer(heads=3, kv_heads=1, dim=6, rot_dims=4, size=9, keep=2, mlp=moe(ff=10)),
                                                       delta_layer(heads=3, kv_heads=1, dim=7, vdim=5, mlp=moe(experts=3, top=2, ff=9)),
                                                       attn2_layer(heads=2, kv_heads=2, dim=6, vdim=5, rot_dims=6, size=11, keep=3)],
-                                                     width=70, vocab=131, bigram=(17, 1000003, 999983)),
+                                                     width=70, vocab=131, bigram=(17, 1000003, 99998300017)),
 }
 
 

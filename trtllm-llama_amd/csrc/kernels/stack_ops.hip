@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void token_shift_kernel(const StackShiftParams
         const int t = blockIdx.x, e = p.tok_entry[t];
         if (p.tok_pos[t] == p.ent_pos0[e])
             return;
-        for (int c = threadIdx.x; c < W; c += 256)
+        for (int c = blockIdx.y * 256 + threadIdx.x; c < W; c += gridDim.y * 256)
         {
             const float a = p.n[(int64_t) t * W + c], b = p.n[(int64_t) (t - 1) * W + c];
             El<DT>::st(p.h, (int64_t) t * W + c, a + (b - a) * p.mu[c]);
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(256) void token_shift_kernel(const StackShiftParams
     const int first = p.ent_first[e], last = first + p.ent_count[e] - 1;
     float* carry = p.carry + (int64_t) p.ent_slot[e] * W;
     const bool fresh = p.ent_pos0[e] == 0;
-    for (int c = threadIdx.x; c < W; c += 256)
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < W; c += gridDim.y * 256)
     {
         const float b = fresh ? 0.f : carry[c];
         const float a = p.n[(int64_t) first * W + c];
@@ -657,7 +657,7 @@ __global__ __launch_bounds__(256) void talk_combine_kernel(const StackAttnParams
     for (int i = threadIdx.x; i < H * H; i += 256)
         tk_s[i] = p.talk[i];
     __syncthreads();
-    for (int oc = threadIdx.x; oc < H * V; oc += 256)
+    for (int oc = blockIdx.y * 256 + threadIdx.x; oc < H * V; oc += gridDim.y * 256)
     {
         const int h = oc / V, ch = oc % V, c = h / per;
         float a = 0.f;
@@ -1114,10 +1114,12 @@ int launch_stack_token_shift(const StackShiftParams& p, hipStream_t stream)
         set_error("stack_token_shift: width %d, or a missing operand", p.width);
         return -1;
     }
+    // few rows (decoding): a row's channels are spread over workgroups
+    const dim3 grid(p.tokens + p.entries, p.tokens >= 128 ? 1 : std::min((p.width + 255) / 256, 16));
     if (p.dtype == DT_BF16)
-        hipLaunchKernelGGL((token_shift_kernel<DT_BF16>), dim3(p.tokens + p.entries), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((token_shift_kernel<DT_BF16>), grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL((token_shift_kernel<DT_FLOAT>), dim3(p.tokens + p.entries), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((token_shift_kernel<DT_FLOAT>), grid, dim3(256), 0, stream, p);
     return launched("stack_token_shift");
 }
 
@@ -1432,10 +1434,12 @@ int launch_stack_talk_combine(const StackAttnParams& p, const void* pairs, hipSt
         set_error("stack_talk_combine: %d heads over %d key/value heads, vdim %d, or a missing operand", p.heads, p.kv_heads, p.vdim);
         return -1;
     }
+    // few rows (decoding): a row's output channels are spread over workgroups
+    const dim3 grid(p.tokens, p.tokens >= 256 ? 1 : std::min((p.heads * p.vdim + 255) / 256, 16));
     if (p.dtype == DT_BF16)
-        hipLaunchKernelGGL((talk_combine_kernel<DT_BF16>), dim3(p.tokens), dim3(256), lds, stream, p, pairs);
+        hipLaunchKernelGGL((talk_combine_kernel<DT_BF16>), grid, dim3(256), lds, stream, p, pairs);
     else
-        hipLaunchKernelGGL((talk_combine_kernel<DT_FLOAT>), dim3(p.tokens), dim3(256), lds, stream, p, pairs);
+        hipLaunchKernelGGL((talk_combine_kernel<DT_FLOAT>), grid, dim3(256), lds, stream, p, pairs);
     return launched("stack_talk_combine");
 }
 

@@ -395,8 +395,17 @@ tllm_stack_t tllm_stack_create(const char* config_text)
     s->norm_offset = (float) getd(s, "norm_offset", 0.0);
     s->streams = geti(s, "streams", 1);
     s->pair_buckets = geti(s, "pair_buckets", 0);
-    s->pair_mul_prev = geti(s, "pair_mul_prev", 0);
-    s->pair_mul_cur = geti(s, "pair_mul_cur", 0);
+    if (s->pair_buckets > 0)
+    {
+        // the multipliers only matter modulo the bucket count: (a m) mod B = (a (m mod B)) mod B, and the kernel's 64-bit products then
+        // have room for any vocabulary
+        auto mod_b = [&](const char* key) {
+            const long long m = std::atoll(gets(s, key, "0").c_str()) % s->pair_buckets;
+            return (int) (m < 0 ? m + s->pair_buckets : m);
+        };
+        s->pair_mul_prev = mod_b("pair_mul_prev");
+        s->pair_mul_cur = mod_b("pair_mul_cur");
+    }
     s->token_shift = geti(s, "token_shift", 0);
     const std::string block = gets(s, "block", "parallel"), residual = gets(s, "residual", "gated");
     s->sequential = block == "sequential";

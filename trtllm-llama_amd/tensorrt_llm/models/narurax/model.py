@@ -62,7 +62,8 @@ class NaruraxConfig(object):
         for i, l in enumerate(self.layers):
             p, m = f'layer.{i}.', l['mixer']
             c[p + 'heads'], c[p + 'kv_heads'] = int(m['heads']), int(m.get('kv_heads', m['heads']))
-            c[p + 'dim'], c[p + 'vdim'] = int(m['dim']), int(m.get('vdim', m['dim']))
+            # an 'attention' layer's values are its keys: their size is the key size
+            c[p + 'dim'], c[p + 'vdim'] = int(m['dim']), int(m['dim'] if l['type'] == 'attention' else m.get('vdim', m['dim']))
             if l['type'] == 'channel_delta':
                 c[p + 'type'], c[p + 'conv'] = 'delta_rule', int(m['conv'])
                 ra, rg = self.ranks.get(i, (self.default_rank(i), self.default_rank(i)))
