@@ -5,6 +5,7 @@
 #include "launch_util.h"
 #include "stack_kernels.h"
 #include <algorithm>
+#include <cstdlib>
 
 namespace tllm
 {
@@ -35,6 +36,21 @@ __device__ __forceinline__ void st_el(void* p, int64_t i, float v)
 __device__ __forceinline__ float softplus_f(float z)
 {
     return z > 20.f ? z : log1pf(expf(z));
+}
+
+// exp(-rate * softplus(z)).  The bfloat16 engine takes the hardware's base-2 exponential and logarithm: their error, relative to
+// 1 + e^z, is a few 1e-7 - far below what rounding the activations leaves; the fp32 engine keeps the library's functions.
+template <int DT>
+__device__ __forceinline__ float decay_of(float rate, float z)
+{
+    if constexpr (DT == DT_BF16)
+    {
+        constexpr float LOG2E = 1.4426950408889634f;
+        const float sp2 = z > 20.f ? z * LOG2E : __builtin_amdgcn_logf(1.f + __builtin_amdgcn_exp2f(z * LOG2E)); // softplus / ln 2
+        return __builtin_amdgcn_exp2f(-rate * sp2);
+    }
+    else
+        return expf(-rate * softplus_f(z));
 }
 
 inline int launched(const char* what)
@@ -80,7 +96,7 @@ __device__ __forceinline__ float slice_sum(float v, int DS)
 // head's columns are independent, so a launch with few (entry, head) pairs cuts them over workgroups; the head norm is a pass of
 // its own (delta_out_kernel).
 template <int DT, int NSZ>
-__global__ __launch_bounds__(256) void delta_scan_kernel(const StackDeltaParams p, int DS, int cols)
+__global__ __launch_bounds__(256) void delta_scan_kernel(const StackDeltaParams p, int DS, int cols, int probe)
 {
     extern __shared__ float sm[];
     const int D = p.dim, V = p.vdim;
@@ -107,53 +123,76 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const StackDeltaParams 
     for (int i = 0; i < NSZ; ++i)
         S[i] = (live && d0 + i < D && p.ent_pos0[e] > 0) ? st[(int64_t) (d0 + i) * V + v] : 0.f;
     constexpr int PF = NSZ < 16 ? NSZ : 16; // elements of the stage a thread fetches per round
+    const int dp_shift = __ffs(DP) - 1;     // DP is a power of two
     const float rate = expf(p.a_log[h]);
     const float q_mul = 1.f / sqrtf((float) D);
+    // A chunk's inputs - per (row, key channel) q, k and the decay's pre-activation, per row the thread's own value and beta - are
+    // fetched into registers with every load in flight at once, and land in the stage behind a barrier.  Every load is unconditional,
+    // at an index clamped into the chunk: a load under a condition would sit in a block of its own with its wait, and the chunk
+    // would pay one memory latency per element instead of one per round.  Where one round holds a whole chunk (the usual case), the
+    // next chunk is fetched while this one is scanned.
+    float rq[PF], rk[PF], ra[PF], rv[DL_RC], rb = 0.f;
+    const int vc = v < V ? v : V - 1;
+    auto fetch = [&](int r0f, int nrf, int base) {
+#pragma unroll
+        for (int j = 0; j < PF; ++j)
+        {
+            const int el = base + j * NT + tid, r = min(el >> dp_shift, nrf - 1), d = min(el & (DP - 1), D - 1);
+            const int64_t t = first + r0f + r;
+            rq[j] = ld_el<DT>(p.x, t * CH + hk * D + d);
+            rk[j] = ld_el<DT>(p.x, t * CH + QK + hk * D + d);
+            ra[j] = p.decay_raw[t * HD + h * D + d] + p.dt_bias[h * D + d];
+        }
+        if (base == 0)
+        {
+#pragma unroll
+            for (int r = 0; r < DL_RC; ++r)
+                rv[r] = ld_el<DT>(p.x, (int64_t) (first + r0f + min(r, nrf - 1)) * CH + 2 * QK + h * V + vc);
+            rb = ld_el<DT>(p.beta_raw, (int64_t) (first + r0f + min(tid, nrf - 1)) * p.ld_beta + h);
+        }
+    };
+    auto land = [&](int nrf, int base) {
+#pragma unroll
+        for (int j = 0; j < PF; ++j)
+        {
+            const int el = base + j * NT + tid;
+            if (el < nrf * DP)
+            {
+                const bool in = (el & (DP - 1)) < D;
+                qs[el] = in ? rq[j] : 0.f;
+                ks[el] = in ? rk[j] : 0.f;
+                gs[el] = in ? ((probe & 2) ? ra[j] : decay_of<DT>(rate, ra[j])) : 0.f;
+            }
+        }
+        if (base == 0)
+        {
+#pragma unroll
+            for (int r = 0; r < DL_RC; ++r)
+                vs[r * NT + tid] = live ? rv[r] : 0.f;
+            if (tid < nrf)
+                bs[tid] = 1.f / (1.f + expf(-rb));
+        }
+    };
+    const bool one_round = DL_RC * DP <= NT * PF && NT >= DL_RC; // uniform
+    if (one_round && count > 0)
+        fetch(0, count < DL_RC ? count : DL_RC, 0);
     for (int r0 = 0; r0 < count; r0 += DL_RC)
     {
         const int nr = count - r0 < DL_RC ? count - r0 : DL_RC;
         __syncthreads(); // the chunk before this one has been read
-        // every thread fetches its share of the chunk's (row, key channel) elements - q, k and the decay's pre-activation - with all
-        // of its loads in flight at once, then the decays are formed and everything lands in the stage
-        for (int base = 0; base < nr * DP; base += NT * PF)
-        {
-            float rq[PF], rk[PF], ra[PF];
-#pragma unroll
-            for (int j = 0; j < PF; ++j)
+        if (one_round)
+            land(nr, 0);
+        else
+            for (int base = 0; base < nr * DP; base += NT * PF)
             {
-                const int el = base + j * NT + tid, r = el / DP, d = el - r * DP;
-                const bool in = el < nr * DP && d < D;
-                const int64_t t = first + r0 + r;
-                rq[j] = in ? ld_el<DT>(p.x, t * CH + hk * D + d) : 0.f;
-                rk[j] = in ? ld_el<DT>(p.x, t * CH + QK + hk * D + d) : 0.f;
-                ra[j] = in ? p.decay_raw[t * HD + h * D + d] + p.dt_bias[h * D + d] : 0.f;
+                fetch(r0, nr, base);
+                land(nr, base);
             }
-#pragma unroll
-            for (int j = 0; j < PF; ++j)
-            {
-                const int el = base + j * NT + tid, r = el / DP, d = el - r * DP;
-                if (el < nr * DP)
-                {
-                    qs[el] = rq[j];
-                    ks[el] = rk[j];
-                    gs[el] = d < D ? expf(-rate * softplus_f(ra[j])) : 0.f;
-                }
-            }
-        }
-        {
-            float rv[DL_RC];
-#pragma unroll
-            for (int r = 0; r < DL_RC; ++r)
-                rv[r] = (live && r < nr) ? ld_el<DT>(p.x, (int64_t) (first + r0 + r) * CH + 2 * QK + h * V + v) : 0.f;
-#pragma unroll
-            for (int r = 0; r < DL_RC; ++r)
-                vs[r * NT + tid] = rv[r];
-        }
-        if (tid < nr)
-            bs[tid] = 1.f / (1.f + expf(-ld_el<DT>(p.beta_raw, (int64_t) (first + r0 + tid) * p.ld_beta + h)));
         __syncthreads();
+        if (one_round && r0 + DL_RC < count)
+            fetch(r0 + DL_RC, count - r0 - DL_RC < DL_RC ? count - r0 - DL_RC : DL_RC, 0);
         // q and k stay as projected in the stage; their unit-norm factors are applied to the sums they enter
-        for (int r = wid; r < nr; r += nwaves)
+        for (int r = wid; r < ((probe & 4) ? 0 : nr); r += nwaves)
         {
             float sq = 0.f, sk = 0.f;
             for (int d = lane; d < D; d += 64)
@@ -170,7 +209,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const StackDeltaParams 
             }
         }
         __syncthreads();
-        for (int r = 0; r < nr; ++r)
+        for (int r = 0; r < ((probe & 1) ? 0 : nr); ++r)
         {
             {
                 // rows of the stage past dim hold zeros and the state rows there stay zero: no guard inside the slices
@@ -285,14 +324,18 @@ int launch_scan(const StackDeltaParams& p, hipStream_t stream)
         cols = (cols + 1) / 2;
     const int threads = (cols * sh.ds + 63) / 64 * 64; // at most 256: cols * slices <= 256, or one column of up to 64 slices
     const dim3 grid(p.entries, p.heads, (p.vdim + cols - 1) / cols);
+    // measurement knob, bits: 1 = no recurrence, 2 = decays without their exponentials, 4 = no unit norms (what is left is the
+    // chunk's traffic and barriers); results are wrong with any of them
+    const char* pv = std::getenv("TLLM_STACK_DELTA_PROBE");
+    const int probe = pv ? std::atoi(pv) : 0;
     const size_t lds = sizeof(float) * ((size_t) 3 * DL_RC * sh.ds * sh.nsz + 3 * DL_RC + (size_t) DL_RC * threads);
     switch (sh.nsz)
     {
-    case 8: hipLaunchKernelGGL((delta_scan_kernel<DT, 8>), grid, dim3(threads), lds, stream, p, sh.ds, cols); break;
-    case 16: hipLaunchKernelGGL((delta_scan_kernel<DT, 16>), grid, dim3(threads), lds, stream, p, sh.ds, cols); break;
+    case 8: hipLaunchKernelGGL((delta_scan_kernel<DT, 8>), grid, dim3(threads), lds, stream, p, sh.ds, cols, probe); break;
+    case 16: hipLaunchKernelGGL((delta_scan_kernel<DT, 16>), grid, dim3(threads), lds, stream, p, sh.ds, cols, probe); break;
     default:
         launch_util::ensure_dynamic_lds(reinterpret_cast<const void*>(&delta_scan_kernel<DT, 32>), 120 * 1024); // raised once, for the largest dim
-        hipLaunchKernelGGL((delta_scan_kernel<DT, 32>), grid, dim3(threads), lds, stream, p, sh.ds, cols);
+        hipLaunchKernelGGL((delta_scan_kernel<DT, 32>), grid, dim3(threads), lds, stream, p, sh.ds, cols, probe);
         break;
     }
     return launched("stack_delta_scan");
