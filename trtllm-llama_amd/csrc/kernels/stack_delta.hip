@@ -122,14 +122,14 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const StackDeltaParams 
 #pragma unroll
     for (int i = 0; i < NSZ; ++i)
         S[i] = (live && d0 + i < D && p.ent_pos0[e] > 0) ? st[(int64_t) (d0 + i) * V + v] : 0.f;
-    constexpr int PF = NSZ < 16 ? NSZ : 16; // elements of the stage a thread fetches per round
+    constexpr int PF = NSZ < 16 ? NSZ : 16; // elements of the stage a thread fetches per pass
     const int dp_shift = __ffs(DP) - 1;     // DP is a power of two
     const float rate = expf(p.a_log[h]);
     const float q_mul = 1.f / sqrtf((float) D);
     // A chunk's inputs - per (row, key channel) q, k and the decay's pre-activation, per row the thread's own value and beta - are
     // fetched into registers with every load in flight at once, and land in the stage behind a barrier.  Every load is unconditional,
     // at an index clamped into the chunk: a load under a condition would sit in a block of its own with its wait, and the chunk
-    // would pay one memory latency per element instead of one per round.  Where one round holds a whole chunk (the usual case), the
+    // would pay one memory latency per element instead of one per pass.  Where one pass holds a whole chunk (the usual case), the
     // next chunk is fetched while this one is scanned.
     float rq[PF], rk[PF], ra[PF], rv[DL_RC], rb = 0.f;
     const int vc = v < V ? v : V - 1;
@@ -173,14 +173,14 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const StackDeltaParams 
                 bs[tid] = 1.f / (1.f + expf(-rb));
         }
     };
-    const bool one_round = DL_RC * DP <= NT * PF && NT >= DL_RC; // uniform
-    if (one_round && count > 0)
+    const bool one_pass = DL_RC * DP <= NT * PF && NT >= DL_RC; // uniform
+    if (one_pass && count > 0)
         fetch(0, count < DL_RC ? count : DL_RC, 0);
     for (int r0 = 0; r0 < count; r0 += DL_RC)
     {
         const int nr = count - r0 < DL_RC ? count - r0 : DL_RC;
         __syncthreads(); // the chunk before this one has been read
-        if (one_round)
+        if (one_pass)
             land(nr, 0);
         else
             for (int base = 0; base < nr * DP; base += NT * PF)
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const StackDeltaParams 
                 land(nr, base);
             }
         __syncthreads();
-        if (one_round && r0 + DL_RC < count)
+        if (one_pass && r0 + DL_RC < count)
             fetch(r0 + DL_RC, count - r0 - DL_RC < DL_RC ? count - r0 - DL_RC : DL_RC, 0);
         // q and k stay as projected in the stage; their unit-norm factors are applied to the sums they enter
         for (int r = wid; r < ((probe & 4) ? 0 : nr); r += nwaves)

@@ -674,7 +674,7 @@ __global__ __launch_bounds__(256) void talk_combine_kernel(const StackAttnParams
 // running maximum and denominator (sink included); the second recomputes the scores, normalises, mixes w'_h = sum_g talk[h, g] w_g per
 // key in the thread that owns it, and multiplies with the values of head h's own key/value head, one thread per output channel of
 // the whole row (heads * vdim / TK_T of them per thread).  One map, softmax weights; any dim, heads * vdim <= TK_T * TK_CPT.
-constexpr int TK_T = 256, TK_CPT = 16, TK_MAXH = 64;
+constexpr int TK_T = 256, TK_CPT = 32, TK_MAXH = 64;
 
 template <int DT>
 __global__ __launch_bounds__(TK_T) void attn_talk_kernel(const StackAttnParams p)
