@@ -60,7 +60,7 @@ typedef struct tllm_stack* tllm_stack_t;
  *     .mlp (gelu_gate: W_down (gelu_tanh(W_gate h) * W_up h) | relu2: W_down relu(W_up h)^2 | moe: .experts experts
  *       W_down (silu(W_gate h) * W_up h) of size .ff plus .identity identity outputs, .top chosen per token among the .route_keep best
  *       of .route_groups equal groups, weights = softmax score * .route_scale; .route_score softmax | sigmoid (every output's
- *       score by itself), .route_weight output | input (the weight multiplies the expert's input row and the outputs are summed as they
+ *       score by itself), .route_weight output | input (an expert runs on weight x row and the outputs are summed as they
  *       are); relu2 and moe in sequential blocks only),
  *     attention: .kv_heads, .maps (1 | 2), .diff (the constant of the second map's weight and of the output scale 1 - diff),
  *       .scale, .softcap (0: none), .head_norm (0 | 1), .rot_dims, .rot_base, .rot_factor (0: no frequency scaling),

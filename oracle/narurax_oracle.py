@@ -235,7 +235,7 @@ margins = None
 
 
 def route(h, w, p, r):
-    """-> (indices [n, top], weights [n, top]): the `top` largest sigmoid scores, lowest index among equals; weights not renormalised."""
+    """-> (indices [n, top], weights [n, top]): the `top` largest sigmoid scores, lowest index among equals; the weights are those scores as they are."""
     z = h @ w[p + 'router'].T
     s = sigmoid(z)
     top = int(r['top'])

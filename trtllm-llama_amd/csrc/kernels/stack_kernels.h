@@ -155,7 +155,7 @@ struct StackAttnParams
     const float* log_r1 = nullptr;
     const float* log_r2 = nullptr;
     // mask: which keys j <= i a row sees.  MASK_WINDOW: i - j < mask_size; MASK_CHUNK: floor(i / mask_size) == floor(j / mask_size);
-    // mask_keep > 0 (windows): the sequence's first mask_keep keys stay visible to every later row, at their true positions
+    // mask_keep > 0 (windows): the sequence's first mask_keep keys stay visible to every later row (each at its own position: nothing about them is shifted)
     int32_t mask = 0, mask_size = 0, mask_keep = 0;
     // weights: WEIGHTS_SOFTMAX, its denominator also holding exp(sink[h]) when sink is set (a logit without key or value);
     // WEIGHTS_SIGMOID: weight = sigmoid(score + wbias[h]) per key, not normalised over keys
@@ -323,7 +323,7 @@ struct StackMoeParams
     int32_t experts = 0, identity = 0, top = 0, group_count = 1, group_keep = 1;
     float scale = 1.f;
     int32_t score = 0;        // ROUTE_SOFTMAX: s = softmax(z) over all outputs; ROUTE_SIGMOID: s = sigmoid(z), every output by itself
-    int32_t weight_input = 0; // 1: the weight multiplies the expert's input row (a_sorted = w h), the outputs are summed unweighted
+    int32_t weight_input = 0; // 1: an expert runs on w h (a_sorted = w h), the outputs are summed unweighted
     const void* h = nullptr;          // [tokens, width]
     const float* router_w = nullptr;  // [experts + identity, width]
     const float* correction = nullptr; // [experts + identity] or null
@@ -346,7 +346,7 @@ int launch_stack_moe_combine(const StackMoeParams& p, const float* y_sorted, flo
 // convolution and silu.  Per token, in fp32:
 //   q <- q / sqrt(sum q^2 + 1e-6) / sqrt(dim),  k <- k / sqrt(sum k^2 + 1e-6),  beta = sigmoid(beta_raw[t, h]),
 //   g[d] = exp(-exp(a_log[h]) * softplus(decay_raw[t, h * dim + d] + dt_bias[h * dim + d])),
-//   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   (the read-out sees the token's own write)
+//   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   (read after the token's own write)
 // launch_stack_delta_scan leaves o in o32 [tokens, heads * vdim]; launch_stack_delta_out turns it into
 //   out[t, h, c] = o / sqrt(mean_c o^2 + eps) * norm_w[c] * sigmoid(gate_raw[t, h * vdim + c]).
 // An entry whose pos0 is 0 starts from a zero state.

@@ -12,7 +12,7 @@ reads its normed input blended with the previous token's (token shift, a learned
                   sigmoid gate.  State and convolution tail live in a state slot
 
 and one feed-forward: a routed mixture of experts W_down (silu(W_gate a) * W_up a), a = s h, with sigmoid router scores s, the `top`
-largest chosen, not renormalised.
+largest chosen and used as they are.
 
 This class reads config.json and the safetensors file and describes the stack to the ragged engine (runtime/stack.py).  What the
 design fixes lives here (which options each mixer kind switches on, the activations); every size and every other constant is read
